@@ -1,0 +1,210 @@
+#!/usr/bin/env python3
+"""Benchmark of the LUT-AMM hot path on one MI355X.
+
+Workload (default): the BERT-base FFN pair as LUT-AMM -- N = 8192 tokens (batch 64 x seq 128),
+768 -> 3072 and 3072 -> 768, sub_vec_len 4, 16 centroids per codebook, int8 LUTs with the
+reference's per-tensor fp32 scale, int32 accumulation, random-init centroids and weights.
+One "step" = one pass of the pair (centroid search + LUT gather for FFN1, then for FFN2) with all
+inputs, LUTs and outputs resident in HBM.  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0                     # MI355X HBM3E
+LDS_PEAK_GBPS = 256 * 256 * 2.4            # 256 CUs x 256 B/clk (ds_read_b128) x 2.4 GHz = 157286 GB/s
+
+
+def synth_amm(rng, K, v, C, M, pimdl, ctx):
+    """Random-init centroids N(0,1) and weight N(0,0.02); LUT built and quantised on the GPU."""
+    CB = K // v
+    cent = rng.standard_normal((CB, C, v)).astype(np.float32)
+    W = (rng.standard_normal((K, M)) * 0.02).astype(np.float32)
+    lut, scales = ctx.lutgen(cent, W, pimdl.LUT_I8, 0)
+    bias = np.zeros(M, np.float32)
+    return cent, lut, scales, bias
+
+
+def algorithmic_bytes(N, K, v, C, M, e=1):
+    CB = K // v
+    ib = 0.5 if C <= 16 else 1.0
+    return {
+        "ccs_hbm": 4 * N * K + 4 * C * K + ib * N * CB,
+        "gather_hbm": ib * N * CB + e * CB * C * M + 4 * N * M + 4 * M,
+        "gather_lds": e * N * CB * M,
+        "eff_ops": 2 * N * K * M,
+    }
+
+
+def cpu_baseline(shapes, N, budget_s=12.0):
+    """The oracle's restatement of the reference's amm_cpu (test_amm.cpp:126-183), timed on this
+    host's cores on a bounded token sample of the same two AMMs."""
+    import oracle
+
+    threads = oracle.max_threads()
+    rng = np.random.default_rng(1)
+    ns = min(N, 1024)
+    work = []
+    for (K, v, C, M) in shapes:
+        CB = K // v
+        x = rng.standard_normal((ns, K)).astype(np.float32)
+        cent = rng.standard_normal((CB, C, v)).astype(np.float32)
+        lut = rng.integers(-128, 128, (CB, C, M)).astype(np.int8)
+        bias = np.zeros(M, np.float32)
+        scratch = (np.empty((ns, CB), np.uint16), np.empty((ns, M), np.int32), np.empty((ns, M), np.float32))
+        work.append((x, cent, lut, bias, v, scratch))
+
+    def one_pass():
+        for x, cent, lut, bias, v, scratch in work:
+            oracle.amm_cpu(x, cent, lut, bias, v, 0.01, 0.0, threads=threads, scratch=scratch)
+
+    one_pass()  # warm-up
+    t0 = time.perf_counter()
+    one_pass()
+    t1 = time.perf_counter() - t0
+    rounds = int(max(2, min(20, budget_s / max(t1, 1e-3))))
+    t0 = time.perf_counter()
+    for _ in range(rounds):
+        one_pass()
+    dt = (time.perf_counter() - t0) / rounds
+    return {"value": ns / dt, "unit": "tokens/s", "cores": threads, "kind": "port",
+            "sample": f"{ns} of {N} tokens through both AMMs of the pair, {rounds} timed rounds after 1 warm-up, "
+                      f"oracle amm_cpu (-O3 -fopenmp, no -march), {dt * 1e3:.1f} ms per round"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--tokens", type=int, default=8192)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU only (the path shards over tokens with no exchange; "
+              "see DESIGN.md); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from __graft_entry__ import load_package
+
+    pimdl = load_package()
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; there is no CPU fallback", file=sys.stderr)
+        sys.exit(3)
+    torch.cuda.set_device(0)
+    ctx = pimdl.Context(0)
+    stream = torch.cuda.current_stream()
+    ctx.set_stream(stream.cuda_stream)
+
+    N, v, C = args.tokens, 4, 16
+    shapes = [(768, v, C, 3072), (3072, v, C, 768)]
+    rng = np.random.default_rng(0)
+    amms = []
+    for (K, vv, CC, M) in shapes:
+        cent, lut, scales, bias = synth_amm(rng, K, vv, CC, M, pimdl, ctx)
+        amms.append(ctx.amm(cent, lut, scales, bias, max_n=N))
+
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    x1 = torch.randn((N, 768), device="cuda", generator=gen, dtype=torch.float32)
+    h = torch.empty((N, 3072), device="cuda", dtype=torch.float32)
+    y = torch.empty((N, 768), device="cuda", dtype=torch.float32)
+    # FFN2's input: GELU of FFN1's output, computed once outside the timed region (the activation
+    # function is not part of the LUT-AMM path)
+    amms[0].run_ptr(x1.data_ptr(), N, h.data_ptr())
+    ctx.synchronize()
+    x2 = torch.nn.functional.gelu(h).contiguous()
+    torch.cuda.synchronize()
+
+    def step():
+        amms[0].run_ptr(x1.data_ptr(), N, h.data_ptr())
+        amms[1].run_ptr(x2.data_ptr(), N, y.data_ptr())
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record(stream)
+    for _ in range(args.steps):
+        step()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ev_ms = e0.elapsed_time(e1) / args.steps
+    ms_per_step = wall_ms
+
+    # per-kernel device times (HIP events on the same stream, each kernel launched on its own)
+    prof = [amms[0].profile(x1.data_ptr(), N, h.data_ptr(), warmup=3, iters=max(10, args.steps)),
+            amms[1].profile(x2.data_ptr(), N, y.data_ptr(), warmup=3, iters=max(10, args.steps))]
+    per_amm = []
+    for name, (K, vv, CC, M), p in zip(("ffn1", "ffn2"), shapes, prof):
+        ab = algorithmic_bytes(N, K, vv, CC, M)
+        per_amm.append({
+            "name": name, "K": K, "M": M, "ccs_ms": p["ccs_ms"], "gather_ms": p["gather_ms"], "amm_ms": p["total_ms"],
+            "tokens_per_s": N / (p["total_ms"] * 1e-3), "eff_gops": ab["eff_ops"] / (p["total_ms"] * 1e-3) / 1e9,
+            "ccs_hbm_gbps": ab["ccs_hbm"] / (p["ccs_ms"] * 1e-3) / 1e9,
+            "ccs_hbm_frac": ab["ccs_hbm"] / (p["ccs_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "gather_lds_gbps": ab["gather_lds"] / (p["gather_ms"] * 1e-3) / 1e9,
+            "gather_lds_frac": ab["gather_lds"] / (p["gather_ms"] * 1e-3) / 1e9 / LDS_PEAK_GBPS,
+            "gather_hbm_gbps": ab["gather_hbm"] / (p["gather_ms"] * 1e-3) / 1e9,
+            "gather_hbm_frac": ab["gather_hbm"] / (p["gather_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "geometry": None,
+        })
+    for pa, amm in zip(per_amm, amms):
+        pa["geometry"] = amm.geometry()
+
+    # dominant kernel: the longer of the two gathers
+    dom = max(per_amm, key=lambda d: d["gather_ms"])
+    K, M = dom["K"], dom["M"]
+    ab = algorithmic_bytes(N, K, v, C, M)
+    _, lds_measured = ctx.diag_bandwidth(copy=False, lds=True)
+    roofline = {
+        "kernel": f"gather_i8_kernel ({dom['name']}: K={K} M={M})",
+        "bound": "lds", "achieved": dom["gather_lds_gbps"], "peak": LDS_PEAK_GBPS, "unit": "GB/s",
+        "frac": dom["gather_lds_frac"],
+        "traffic": None,
+        "algorithmic_bytes_per_launch": ab["gather_lds"],
+        "avg_launch_ms": dom["gather_ms"],
+        "lds_peak_measured_gbps": lds_measured,
+        "frac_of_measured_lds_peak": dom["gather_lds_gbps"] / lds_measured if lds_measured else None,
+        "hbm": {"achieved": dom["gather_hbm_gbps"], "peak": HBM_PEAK_GBPS, "frac": dom["gather_hbm_frac"],
+                "algorithmic_bytes_per_launch": ab["gather_hbm"]},
+    }
+
+    total_eff_ops = sum(algorithmic_bytes(N, K_, v, C, M_)["eff_ops"] for (K_, _, _, M_) in shapes)
+    result = {
+        "metric": "LUT-AMM tokens/s (BERT-base FFN pair, N=8192)",
+        "value": N / (ms_per_step * 1e-3),
+        "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "i8", "data": "synthetic",
+        "config": {"workload": "BERT-base FFN pair as LUT-AMM: N=8192 (64x128) fp32 activations N(0,1); "
+                               "768->3072 and 3072->768, vec_len=4, 16 centroids/codebook, int8 LUT with the "
+                               "reference's per-tensor fp32 scale, int32 accumulate, random-init centroids/weights",
+                   "tokens": N, "vec_len": v, "num_centroid": C},
+        "eff_gops": total_eff_ops / (ms_per_step * 1e-3) / 1e9,
+        "device_ms_per_step": ev_ms,
+        "per_amm": per_amm,
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(shapes, N)
+    for a in amms:
+        a.close()
+    ctx.close()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

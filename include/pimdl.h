@@ -1,0 +1,181 @@
+/*
+ * pimdl.h -- C ABI of the MI355X (gfx950) LUT-AMM engine.
+ *
+ * One data-parallel path: closest-centroid search over activation sub-vectors, gather of
+ * pre-computed centroid x weight LUT rows by those indices, sum across codebooks, de-quantise.
+ * Plain pointers and sizes only; no C++ or torch types cross this boundary.  Every entry point
+ * returns PIMDL_OK (0) or a negative pimdl_status; pimdl_last_error() gives the text.
+ *
+ * Each entry point names the interface of the reference (PIM-DL, paths under its
+ * inference-engine/ or model-calibration/ trees) that it replaces.
+ *
+ * Conventions
+ *   N tokens, K = input_feature_len, v = sub_vec_len, CB = K / v codebooks, C = num_centroid,
+ *   M = output_feature_len.
+ *   centroids  fp32 [CB][C][v]                     (src/host/index_calc_host.cpp:23)
+ *   LUT        int8 or fp32 [CB][C][M], canonical  (test/test_amm.cpp:173; the .npz
+ *                                                   "<op>.lut.tensor" written by
+ *                                                   pim_weight_converter.py:89-94)
+ *   input      fp32 [N][K] row-major, output fp32 [N][M] row-major.
+ *   "dev" pointers are HIP device pointers; "host" pointers are ordinary host memory.
+ *   pimdl_amm_run() accepts either kind for input and output and finds out which by itself.
+ */
+#ifndef PIMDL_H
+#define PIMDL_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(PIMDL_BUILD)
+#define PIMDL_API __attribute__((visibility("default")))
+#else
+#define PIMDL_API
+#endif
+
+typedef enum pimdl_status {
+    PIMDL_OK = 0,
+    PIMDL_ERR_INVALID = -1,     /* null pointer, zero size, K % v != 0, n > max_n ... */
+    PIMDL_ERR_UNSUPPORTED = -2, /* shape outside what the kernels are built for */
+    PIMDL_ERR_HIP = -3,         /* a HIP runtime call failed (text has hipGetErrorString) */
+    PIMDL_ERR_NOMEM = -4,
+    PIMDL_ERR_NO_DEVICE = -5    /* no gfx950 device visible: there is no CPU fallback */
+} pimdl_status;
+
+typedef enum pimdl_lut_dtype { PIMDL_LUT_I8 = 0, PIMDL_LUT_F32 = 1 } pimdl_lut_dtype;
+
+/* How the epilogue adds the scalar LUT bias (both exist in the reference and differ unless
+ * the bias is 0, which is all its converter ever writes):
+ *   PIMDL_BIAS_ONCE       out = acc*scale + lut_bias      + bias[f]   test/test_amm.cpp:181
+ *   PIMDL_BIAS_TIMES_CB   out = acc*scale + lut_bias*CB   + bias[f]   src/host/pim_lut_host.cpp:201 */
+typedef enum pimdl_bias_mode { PIMDL_BIAS_ONCE = 0, PIMDL_BIAS_TIMES_CB = 1 } pimdl_bias_mode;
+
+typedef struct pimdl_ctx pimdl_ctx; /* one device + one stream + scratch */
+typedef struct pimdl_amm pimdl_amm; /* one linear layer's centroids + LUT + bias, resident in HBM */
+
+/* Shape and numeric mode of one AMM operator.  Mirrors the shape fields of IndexCalcParams and
+ * LUTParams (src/host/defines.h:12-50); the DPU tiling fields have no meaning on a GPU. */
+typedef struct pimdl_amm_desc {
+    uint32_t max_n;             /* largest N a run may pass */
+    uint32_t input_feature_len; /* K */
+    uint32_t sub_vec_len;       /* v */
+    uint32_t num_centroid;      /* C, 2..256 */
+    uint32_t output_feature_len;/* M */
+    uint32_t lut_dtype;         /* pimdl_lut_dtype */
+    uint32_t scale_group;       /* int8 only. 0: one scale for the tensor (the reference,
+                                   LUTParams.scale).  g > 0 (extension): one scale per g
+                                   consecutive codebooks, int32 inside a group, fp32 across. */
+    uint32_t bias_mode;         /* pimdl_bias_mode */
+    float lut_bias;             /* LUTParams.bias */
+} pimdl_amm_desc;
+
+/* Timing of the last profiled run, milliseconds on the device (HIP events on the context's
+ * stream, averaged over `iters` launches of each kernel on its own). */
+typedef struct pimdl_amm_timing {
+    float ccs_ms;    /* closest-centroid search kernel */
+    float gather_ms; /* LUT gather-accumulate (+ epilogue) kernel */
+    float total_ms;  /* both, back to back, as pimdl_amm_run issues them */
+} pimdl_amm_timing;
+
+/* ---- context ---------------------------------------------------------------------------
+ * Replaces allocate_dpu / allocate_rank / load_binary / free_dpu_set
+ * (src/host/dpu_common.h:11-54): the opaque device handle every call takes. */
+PIMDL_API int pimdl_init(int device, pimdl_ctx** out);
+PIMDL_API int pimdl_destroy(pimdl_ctx* ctx);
+/* Text of the last error on this context (or of the last failed pimdl_init when ctx is NULL). */
+PIMDL_API const char* pimdl_last_error(const pimdl_ctx* ctx);
+/* Run this context's kernels on a caller-owned hipStream_t (NULL: back to the context's own).
+ * Lets a caller that already has a stream (e.g. torch's current stream) order and time work. */
+PIMDL_API int pimdl_set_stream(pimdl_ctx* ctx, void* hip_stream);
+PIMDL_API int pimdl_synchronize(pimdl_ctx* ctx);
+
+/* ---- operator: upload once, run many times ---------------------------------------------
+ * Replaces prepare_lut_table (src/host/pim_lut_host.cpp:26-37), which re-sends the LUT to the
+ * DPUs on every call, and the per-op load_binary before each amm_host in
+ * src/host/transformer_layer.cpp:300,430,499,555.  All pointers are HOST pointers; the data is
+ * copied (the LUT is re-tiled into column blocks for LDS staging) and may be freed on return.
+ *   centroids  fp32 [CB][C][v]
+ *   lut        int8 or fp32 [CB][C][M], canonical layout
+ *   scales     int8: 1 float (scale_group 0) or ceil(CB/scale_group) floats; fp32 LUT: NULL
+ *   bias       fp32 [M] or NULL (treated as zeros)                                        */
+PIMDL_API int pimdl_amm_create(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const float* centroids,
+                               const void* lut, const float* scales, const float* bias,
+                               pimdl_amm** out);
+PIMDL_API int pimdl_amm_destroy(pimdl_amm* amm);
+
+/* The AMM itself.  Replaces amm_host (src/host/amm_host.h:8-10, amm_host.cpp:10-30) =
+ * index_calculation + pim_lut, with row-major input and output.
+ *   in   fp32 [n][K], host or device
+ *   out  fp32 [n][M], host or device
+ * Synchronous for host pointers.  For device pointers the kernels are queued on the context's
+ * stream and the call returns at once; use pimdl_synchronize() or stream ordering. */
+PIMDL_API int pimdl_amm_run(pimdl_amm* amm, const float* in, uint32_t n, float* out);
+
+/* As pimdl_amm_run, plus the two intermediates that make the bit-exact claims checkable:
+ *   idx_out  host uint16 [n][CB] centroid ids (what index_calculation writes under the
+ *            identity tiling, src/host/index_calc_host.cpp:41-49), or NULL
+ *   acc_out  host int32 [n][M] accumulators before de-quantisation (int8 LUT, scale_group 0
+ *            only; the DPU's output_data, src/host/pim_lut_host.cpp:173-181), or NULL
+ * Always synchronous. */
+PIMDL_API int pimdl_amm_run_debug(pimdl_amm* amm, const float* in, uint32_t n, float* out,
+                                  uint16_t* idx_out, int32_t* acc_out);
+
+/* Runs the two kernels `iters` times each on device-resident buffers and reports the average
+ * device time of each.  in/out must be DEVICE pointers. */
+PIMDL_API int pimdl_amm_profile(pimdl_amm* amm, const float* in_dev, uint32_t n, float* out_dev,
+                                uint32_t warmup, uint32_t iters, pimdl_amm_timing* timing);
+
+/* ---- the two halves on their own ---------------------------------------------------------
+ * pimdl_index_calculation replaces index_calculation (src/host/index_calc_host.h:5,
+ * index_calc_host.cpp:8-53).  in is host or device fp32 [n][K]; idx_out is HOST uint16, written
+ * at the reference's tiled offset (index_calc_host.cpp:41-49); n_stile_size == n and
+ * cb_mtile_size == CB give row-major [n][CB].  Uses the operator's resident centroids. */
+PIMDL_API int pimdl_index_calculation(pimdl_amm* amm, const float* in, uint32_t n,
+                                      uint16_t* idx_out, uint32_t n_stile_size,
+                                      uint32_t cb_mtile_size);
+/* pimdl_lut_gather replaces pim_lut (src/host/pim_lut_host.h:13-14, pim_lut_host.cpp:121-222):
+ * idx is HOST uint16 row-major [n][CB] holding centroid ids; out is host or device fp32 [n][M]. */
+PIMDL_API int pimdl_lut_gather(pimdl_amm* amm, const uint16_t* idx, uint32_t n, float* out);
+
+/* ---- LUT construction ----------------------------------------------------------------------
+ * Replaces model-calibration/pim_weight_converter.py:82-91 (bmm of centroids with the weight)
+ * and lut_quant (:21-35).  All pointers are HOST pointers.
+ *   centroids fp32 [CB][C][v];  weight fp32 [K][M] (the transposed nn.Linear weight)
+ *   lut_dtype PIMDL_LUT_F32: lut_out fp32 [CB][C][M], scales_out untouched
+ *   lut_dtype PIMDL_LUT_I8 : lut_out int8 [CB][C][M]; scale_group 0: scales_out[0] =
+ *             max|lut|/127 over the tensor (the reference); g > 0: one per g codebooks. */
+PIMDL_API int pimdl_lutgen(pimdl_ctx* ctx, const float* centroids, const float* weight,
+                           uint32_t num_codebook, uint32_t num_centroid, uint32_t sub_vec_len,
+                           uint32_t output_feature_len, uint32_t lut_dtype, uint32_t scale_group,
+                           void* lut_out, float* scales_out);
+
+/* ---- introspection ---------------------------------------------------------------------------
+ * No reference counterpart: figures a benchmark needs to place a kernel on its roofline. */
+typedef struct pimdl_device_info {
+    char name[64];
+    char arch[32];            /* "gfx950..." */
+    uint32_t compute_units;
+    uint32_t clock_khz;
+    uint32_t lds_bytes_per_cu;
+    uint64_t hbm_bytes;
+} pimdl_device_info;
+PIMDL_API int pimdl_get_device_info(pimdl_ctx* ctx, pimdl_device_info* info);
+/* Geometry the operator's kernels were launched with (for documentation of a measurement). */
+typedef struct pimdl_amm_geometry {
+    uint32_t num_codebook, num_codebook_padded, idx_bits, idx_row_bytes;
+    uint32_t col_block, row_pitch, cb_per_slice, lds_bytes, tokens_per_wg, gather_threads;
+    uint32_t ccs_tokens_per_wg, ccs_cb_per_wg, ccs_threads, ccs_lds_bytes;
+} pimdl_amm_geometry;
+PIMDL_API int pimdl_amm_get_geometry(const pimdl_amm* amm, pimdl_amm_geometry* g);
+/* Achieved bandwidth, GB/s, of (a) a plain device-to-device copy kernel of `bytes` bytes and
+ * (b) a ds_read_b128 loop that keeps every CU's LDS busy.  Either pointer may be NULL. */
+PIMDL_API int pimdl_diag_bandwidth(pimdl_ctx* ctx, uint64_t bytes, float* copy_gbps,
+                                   float* lds_gbps);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PIMDL_H */

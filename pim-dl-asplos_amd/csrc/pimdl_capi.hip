@@ -1,0 +1,492 @@
+// C ABI of libpimdl (see include/pimdl.h).  Host-side plumbing only: shape checks, uploads,
+// scratch buffers, pointer classification, kernel sequencing.  There is no CPU compute path:
+// without a gfx950 device pimdl_init fails and nothing else can be called.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <vector>
+
+#include "pimdl_internal.h"
+
+namespace pimdl {
+
+static thread_local std::string g_init_error;
+
+int set_error(Ctx* ctx, int code, const char* fmt, ...)
+{
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    if (ctx) ctx->err = buf;
+    else g_init_error = buf;
+    return code;
+}
+
+int hip_check(Ctx* ctx, hipError_t e, const char* what)
+{
+    if (e == hipSuccess) return PIMDL_OK;
+    return set_error(ctx, e == hipErrorOutOfMemory ? PIMDL_ERR_NOMEM : PIMDL_ERR_HIP, "%s: %s", what,
+                     hipGetErrorString(e));
+}
+
+static bool is_device_ptr(const void* p)
+{
+    hipPointerAttribute_t attr;
+    memset(&attr, 0, sizeof(attr));
+    hipError_t e = hipPointerGetAttributes(&attr, p);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();  // ordinary host memory is reported as an error; clear it
+        return false;
+    }
+    return attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged;
+}
+
+template <typename T>
+static int ensure(Ctx* ctx, T** buf, size_t* have, size_t need, const char* what)
+{
+    if (*have >= need) return PIMDL_OK;
+    if (*buf) {
+        int rc = hip_check(ctx, hipStreamSynchronize(ctx->stream), "sync before scratch regrow");
+        if (rc) return rc;
+        (void)hipFree(*buf);
+        *buf = nullptr;
+        *have = 0;
+    }
+    int rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(buf), need), what);
+    if (rc) return rc;
+    *have = need;
+    return PIMDL_OK;
+}
+
+static int activate(Ctx* ctx) { return hip_check(ctx, hipSetDevice(ctx->device), "hipSetDevice"); }
+
+// input/output staging common to run / run_debug / the two halves
+struct IoPlan {
+    const float* d_in;
+    float* d_out;
+    bool out_is_host;
+};
+
+static int stage_input(Ctx* ctx, const AmmGeom& g, const float* in, uint32_t n, const float** d_in)
+{
+    if (is_device_ptr(in)) {
+        *d_in = in;
+        return PIMDL_OK;
+    }
+    const size_t bytes = (size_t)n * g.K * sizeof(float);
+    int rc = ensure(ctx, &ctx->d_in, &ctx->in_bytes, bytes, "hipMalloc(input scratch)");
+    if (rc) return rc;
+    rc = hip_check(ctx, hipMemcpyAsync(ctx->d_in, in, bytes, hipMemcpyHostToDevice, ctx->stream), "H2D input");
+    *d_in = ctx->d_in;
+    return rc;
+}
+
+static int stage_output(Ctx* ctx, const AmmGeom& g, float* out, uint32_t n, float** d_out, bool* host)
+{
+    if (is_device_ptr(out)) {
+        *d_out = out;
+        *host = false;
+        return PIMDL_OK;
+    }
+    const size_t bytes = (size_t)n * g.M * sizeof(float);
+    int rc = ensure(ctx, &ctx->d_out, &ctx->out_bytes, bytes, "hipMalloc(output scratch)");
+    *d_out = ctx->d_out;
+    *host = true;
+    return rc;
+}
+
+static int finish_output(Ctx* ctx, const AmmGeom& g, float* out, uint32_t n, bool host)
+{
+    if (!host) return PIMDL_OK;
+    int rc = hip_check(ctx, hipMemcpyAsync(out, ctx->d_out, (size_t)n * g.M * sizeof(float), hipMemcpyDeviceToHost,
+                                           ctx->stream), "D2H output");
+    if (rc) return rc;
+    return hip_check(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+}
+
+static int check_run_args(Amm* amm, const void* a, const void* b, uint32_t n)
+{
+    if (!amm) return PIMDL_ERR_INVALID;
+    if (!a || !b) return set_error(amm->ctx, PIMDL_ERR_INVALID, "null buffer");
+    if (n > amm->desc.max_n)
+        return set_error(amm->ctx, PIMDL_ERR_INVALID, "n=%u exceeds max_n=%u of this operator", n, amm->desc.max_n);
+    return activate(amm->ctx);
+}
+
+template <typename T>
+static void retile_lut(const T* lut, T* tiled, const AmmGeom& g, uint32_t row_elems)
+{
+    // canonical [CB][C][M] -> [M_pad/row_elems][CB_pad][C_tile][row_elems], zero padded
+    const uint32_t nblk = g.M_pad / row_elems;
+    for (uint32_t b = 0; b < nblk; ++b)
+        for (uint32_t cb = 0; cb < g.CB; ++cb)
+            for (uint32_t c = 0; c < g.C; ++c) {
+                const T* src = lut + ((size_t)cb * g.C + c) * g.M + (size_t)b * row_elems;
+                T* dst = tiled + (((size_t)b * g.CB_pad + cb) * g.C_tile + c) * row_elems;
+                const uint32_t cnt = (b + 1) * row_elems <= g.M ? row_elems : g.M - b * row_elems;
+                memcpy(dst, src, sizeof(T) * cnt);
+            }
+}
+
+}  // namespace pimdl
+
+using namespace pimdl;
+
+struct pimdl_ctx : Ctx {};
+struct pimdl_amm : Amm {};
+
+extern "C" {
+
+int pimdl_init(int device, pimdl_ctx** out)
+{
+    if (!out) return set_error(nullptr, PIMDL_ERR_INVALID, "pimdl_init: out is null");
+    *out = nullptr;
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count == 0) {
+        (void)hipGetLastError();
+        return set_error(nullptr, PIMDL_ERR_NO_DEVICE,
+                         "pimdl_init: no HIP device visible (%s); this library has no CPU fallback",
+                         e == hipSuccess ? "device count 0" : hipGetErrorString(e));
+    }
+    if (device < 0 || device >= count)
+        return set_error(nullptr, PIMDL_ERR_INVALID, "pimdl_init: device %d out of range (0..%d)", device, count - 1);
+    pimdl_ctx* ctx = new pimdl_ctx();
+    ctx->device = device;
+    ctx->own_stream = nullptr;
+    ctx->stream = nullptr;
+    ctx->d_in = nullptr; ctx->in_bytes = 0;
+    ctx->d_out = nullptr; ctx->out_bytes = 0;
+    ctx->d_idx = nullptr; ctx->idx_bytes = 0;
+    ctx->d_acc = nullptr; ctx->acc_bytes = 0;
+    ctx->d_idx16 = nullptr; ctx->idx16_bytes = 0;
+    for (auto& ev : ctx->ev) ev = nullptr;
+    int rc = hip_check(ctx, hipSetDevice(device), "hipSetDevice");
+    if (!rc) rc = hip_check(ctx, hipGetDeviceProperties(&ctx->prop, device), "hipGetDeviceProperties");
+    if (!rc && strncmp(ctx->prop.gcnArchName, "gfx950", 6) != 0)
+        rc = set_error(ctx, PIMDL_ERR_UNSUPPORTED, "pimdl_init: device %d is %s; the kernels are built for gfx950 only",
+                       device, ctx->prop.gcnArchName);
+    if (!rc) rc = hip_check(ctx, hipStreamCreate(&ctx->own_stream), "hipStreamCreate");
+    for (auto& ev : ctx->ev)
+        if (!rc) rc = hip_check(ctx, hipEventCreate(&ev), "hipEventCreate");
+    if (rc) {
+        g_init_error = ctx->err;
+        pimdl_destroy(ctx);
+        return rc;
+    }
+    ctx->stream = ctx->own_stream;
+    *out = ctx;
+    return PIMDL_OK;
+}
+
+int pimdl_destroy(pimdl_ctx* ctx)
+{
+    if (!ctx) return PIMDL_OK;
+    (void)hipSetDevice(ctx->device);
+    if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    (void)hipFree(ctx->d_in);
+    (void)hipFree(ctx->d_out);
+    (void)hipFree(ctx->d_idx);
+    (void)hipFree(ctx->d_acc);
+    (void)hipFree(ctx->d_idx16);
+    for (auto& ev : ctx->ev)
+        if (ev) (void)hipEventDestroy(ev);
+    if (ctx->own_stream) (void)hipStreamDestroy(ctx->own_stream);
+    delete ctx;
+    return PIMDL_OK;
+}
+
+const char* pimdl_last_error(const pimdl_ctx* ctx) { return ctx ? ctx->err.c_str() : g_init_error.c_str(); }
+
+int pimdl_set_stream(pimdl_ctx* ctx, void* hip_stream)
+{
+    if (!ctx) return PIMDL_ERR_INVALID;
+    int rc = activate(ctx);
+    if (rc) return rc;
+    rc = hip_check(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize(old stream)");
+    ctx->stream = hip_stream ? reinterpret_cast<hipStream_t>(hip_stream) : ctx->own_stream;
+    return rc;
+}
+
+int pimdl_synchronize(pimdl_ctx* ctx)
+{
+    if (!ctx) return PIMDL_ERR_INVALID;
+    int rc = activate(ctx);
+    if (rc) return rc;
+    return hip_check(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+}
+
+int pimdl_amm_create(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const float* centroids, const void* lut,
+                     const float* scales, const float* bias, pimdl_amm** out)
+{
+    if (!ctx) return PIMDL_ERR_INVALID;
+    if (!desc || !centroids || !lut || !out) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_create: null argument");
+    *out = nullptr;
+    int rc = activate(ctx);
+    if (rc) return rc;
+    AmmGeom g;
+    memset(&g, 0, sizeof(g));
+    std::string why;
+    if (!plan_geometry(*desc, &g, &why)) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_create: %s", why.c_str());
+    const bool i8 = desc->lut_dtype == PIMDL_LUT_I8;
+    if (i8 && !scales) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_create: int8 LUT needs scales");
+    if (i8 && desc->scale_group != 0)
+        return set_error(ctx, PIMDL_ERR_UNSUPPORTED,
+                         "pimdl_amm_create: scale_group=%u: only the per-tensor scale (0) is implemented",
+                         desc->scale_group);
+
+    pimdl_amm* a = new pimdl_amm();
+    a->ctx = ctx;
+    a->desc = *desc;
+    a->g = g;
+    a->d_centroids = nullptr;
+    a->d_lut = nullptr;
+    a->d_scales = nullptr;
+    a->d_bias = nullptr;
+    a->nscales = i8 ? 1 : 0;
+    a->h_scale0 = i8 ? scales[0] : 1.0f;
+
+    const size_t cent_bytes = (size_t)g.CB * g.C * g.v * sizeof(float);
+    const size_t elem = i8 ? 1 : 4;
+    const uint32_t row_elems = g.col_block;
+    a->lut_bytes = (size_t)g.M_pad * g.CB_pad * g.C_tile * elem;
+    std::vector<unsigned char> tiled;
+    try {
+        tiled.assign(a->lut_bytes, 0);
+    } catch (...) {
+        delete a;
+        return set_error(ctx, PIMDL_ERR_NOMEM, "pimdl_amm_create: host staging of %zu bytes failed", a->lut_bytes);
+    }
+    if (i8) retile_lut(reinterpret_cast<const int8_t*>(lut), reinterpret_cast<int8_t*>(tiled.data()), g, row_elems);
+    else retile_lut(reinterpret_cast<const float*>(lut), reinterpret_cast<float*>(tiled.data()), g, row_elems);
+
+    rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&a->d_centroids), cent_bytes), "hipMalloc(centroids)");
+    if (!rc) rc = hip_check(ctx, hipMalloc(&a->d_lut, a->lut_bytes), "hipMalloc(lut)");
+    if (!rc) rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&a->d_bias), (size_t)g.M * sizeof(float)), "hipMalloc(bias)");
+    if (!rc && i8) rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&a->d_scales), sizeof(float) * a->nscales), "hipMalloc(scales)");
+    if (!rc) rc = hip_check(ctx, hipMemcpy(a->d_centroids, centroids, cent_bytes, hipMemcpyHostToDevice), "H2D centroids");
+    if (!rc) rc = hip_check(ctx, hipMemcpy(a->d_lut, tiled.data(), a->lut_bytes, hipMemcpyHostToDevice), "H2D lut");
+    if (!rc) {
+        if (bias) rc = hip_check(ctx, hipMemcpy(a->d_bias, bias, (size_t)g.M * sizeof(float), hipMemcpyHostToDevice), "H2D bias");
+        else rc = hip_check(ctx, hipMemset(a->d_bias, 0, (size_t)g.M * sizeof(float)), "memset bias");
+    }
+    if (!rc && i8) rc = hip_check(ctx, hipMemcpy(a->d_scales, scales, sizeof(float) * a->nscales, hipMemcpyHostToDevice), "H2D scales");
+    if (rc) {
+        pimdl_amm_destroy(a);
+        return rc;
+    }
+    *out = a;
+    return PIMDL_OK;
+}
+
+int pimdl_amm_destroy(pimdl_amm* a)
+{
+    if (!a) return PIMDL_OK;
+    (void)hipSetDevice(a->ctx->device);
+    (void)hipStreamSynchronize(a->ctx->stream);
+    (void)hipFree(a->d_centroids);
+    (void)hipFree(a->d_lut);
+    (void)hipFree(a->d_scales);
+    (void)hipFree(a->d_bias);
+    delete a;
+    return PIMDL_OK;
+}
+
+int pimdl_amm_run(pimdl_amm* a, const float* in, uint32_t n, float* out)
+{
+    int rc = check_run_args(a, in, out, n);
+    if (rc || n == 0) return rc;
+    Ctx* ctx = a->ctx;
+    const float* d_in;
+    float* d_out;
+    bool out_host;
+    if ((rc = stage_input(ctx, a->g, in, n, &d_in))) return rc;
+    if ((rc = stage_output(ctx, a->g, out, n, &d_out, &out_host))) return rc;
+    if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, (size_t)n * a->g.idx_row_bytes, "hipMalloc(index scratch)"))) return rc;
+    if ((rc = launch_ccs(ctx, a->g, d_in, a->d_centroids, ctx->d_idx, n))) return rc;
+    if ((rc = launch_gather(ctx, *a, ctx->d_idx, d_out, nullptr, n))) return rc;
+    return finish_output(ctx, a->g, out, n, out_host);
+}
+
+int pimdl_amm_run_debug(pimdl_amm* a, const float* in, uint32_t n, float* out, uint16_t* idx_out, int32_t* acc_out)
+{
+    int rc = check_run_args(a, in, out, n);
+    if (rc || n == 0) return rc;
+    Ctx* ctx = a->ctx;
+    const AmmGeom& g = a->g;
+    if (acc_out && a->desc.lut_dtype != PIMDL_LUT_I8)
+        return set_error(ctx, PIMDL_ERR_INVALID, "acc_out is only defined for int8 LUTs");
+    const float* d_in;
+    float* d_out;
+    bool out_host;
+    if ((rc = stage_input(ctx, g, in, n, &d_in))) return rc;
+    if ((rc = stage_output(ctx, g, out, n, &d_out, &out_host))) return rc;
+    if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, (size_t)n * g.idx_row_bytes, "hipMalloc(index scratch)"))) return rc;
+    if (acc_out && (rc = ensure(ctx, &ctx->d_acc, &ctx->acc_bytes, (size_t)n * g.M * 4, "hipMalloc(acc scratch)"))) return rc;
+    if (idx_out && (rc = ensure(ctx, &ctx->d_idx16, &ctx->idx16_bytes, (size_t)n * g.CB * 2, "hipMalloc(idx16 scratch)"))) return rc;
+    if ((rc = launch_ccs(ctx, g, d_in, a->d_centroids, ctx->d_idx, n))) return rc;
+    if ((rc = launch_gather(ctx, *a, ctx->d_idx, d_out, acc_out ? ctx->d_acc : nullptr, n))) return rc;
+    if (idx_out) {
+        if ((rc = launch_unpack_idx(ctx, g, ctx->d_idx, ctx->d_idx16, n, n, g.CB))) return rc;
+        if ((rc = hip_check(ctx, hipMemcpyAsync(idx_out, ctx->d_idx16, (size_t)n * g.CB * 2, hipMemcpyDeviceToHost, ctx->stream), "D2H idx"))) return rc;
+    }
+    if (acc_out &&
+        (rc = hip_check(ctx, hipMemcpyAsync(acc_out, ctx->d_acc, (size_t)n * g.M * 4, hipMemcpyDeviceToHost, ctx->stream), "D2H acc")))
+        return rc;
+    if ((rc = finish_output(ctx, g, out, n, out_host))) return rc;
+    return hip_check(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+}
+
+int pimdl_amm_profile(pimdl_amm* a, const float* in_dev, uint32_t n, float* out_dev, uint32_t warmup, uint32_t iters,
+                      pimdl_amm_timing* timing)
+{
+    int rc = check_run_args(a, in_dev, out_dev, n);
+    if (rc) return rc;
+    Ctx* ctx = a->ctx;
+    if (!timing || !iters || !n) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_profile: bad arguments");
+    if (!is_device_ptr(in_dev) || !is_device_ptr(out_dev))
+        return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_profile: in/out must be device pointers");
+    if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, (size_t)n * a->g.idx_row_bytes, "hipMalloc(index scratch)"))) return rc;
+    for (uint32_t i = 0; i < warmup; ++i) {
+        if ((rc = launch_ccs(ctx, a->g, in_dev, a->d_centroids, ctx->d_idx, n))) return rc;
+        if ((rc = launch_gather(ctx, *a, ctx->d_idx, out_dev, nullptr, n))) return rc;
+    }
+    float ms[3] = {0, 0, 0};
+    for (int phase = 0; phase < 3; ++phase) {
+        if ((rc = hip_check(ctx, hipEventRecord(ctx->ev[0], ctx->stream), "hipEventRecord"))) return rc;
+        for (uint32_t i = 0; i < iters; ++i) {
+            if (phase != 1 && (rc = launch_ccs(ctx, a->g, in_dev, a->d_centroids, ctx->d_idx, n))) return rc;
+            if (phase != 0 && (rc = launch_gather(ctx, *a, ctx->d_idx, out_dev, nullptr, n))) return rc;
+        }
+        if ((rc = hip_check(ctx, hipEventRecord(ctx->ev[1], ctx->stream), "hipEventRecord"))) return rc;
+        if ((rc = hip_check(ctx, hipEventSynchronize(ctx->ev[1]), "hipEventSynchronize"))) return rc;
+        if ((rc = hip_check(ctx, hipEventElapsedTime(&ms[phase], ctx->ev[0], ctx->ev[1]), "hipEventElapsedTime"))) return rc;
+    }
+    timing->ccs_ms = ms[0] / iters;
+    timing->gather_ms = ms[1] / iters;
+    timing->total_ms = ms[2] / iters;
+    return PIMDL_OK;
+}
+
+int pimdl_index_calculation(pimdl_amm* a, const float* in, uint32_t n, uint16_t* idx_out, uint32_t n_stile_size,
+                            uint32_t cb_mtile_size)
+{
+    int rc = check_run_args(a, in, idx_out, n);
+    if (rc || n == 0) return rc;
+    Ctx* ctx = a->ctx;
+    const AmmGeom& g = a->g;
+    if (!n_stile_size || !cb_mtile_size || n % n_stile_size || g.CB % cb_mtile_size)
+        return set_error(ctx, PIMDL_ERR_INVALID, "n_stile_size must divide n and cb_mtile_size must divide num_codebook");
+    const float* d_in;
+    if ((rc = stage_input(ctx, g, in, n, &d_in))) return rc;
+    if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, (size_t)n * g.idx_row_bytes, "hipMalloc(index scratch)"))) return rc;
+    if ((rc = ensure(ctx, &ctx->d_idx16, &ctx->idx16_bytes, (size_t)n * g.CB * 2, "hipMalloc(idx16 scratch)"))) return rc;
+    if ((rc = launch_ccs(ctx, g, d_in, a->d_centroids, ctx->d_idx, n))) return rc;
+    if ((rc = launch_unpack_idx(ctx, g, ctx->d_idx, ctx->d_idx16, n, n_stile_size, cb_mtile_size))) return rc;
+    if ((rc = hip_check(ctx, hipMemcpyAsync(idx_out, ctx->d_idx16, (size_t)n * g.CB * 2, hipMemcpyDeviceToHost, ctx->stream), "D2H idx"))) return rc;
+    return hip_check(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+}
+
+int pimdl_lut_gather(pimdl_amm* a, const uint16_t* idx, uint32_t n, float* out)
+{
+    int rc = check_run_args(a, idx, out, n);
+    if (rc || n == 0) return rc;
+    Ctx* ctx = a->ctx;
+    const AmmGeom& g = a->g;
+    float* d_out;
+    bool out_host;
+    if ((rc = stage_output(ctx, g, out, n, &d_out, &out_host))) return rc;
+    if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, (size_t)n * g.idx_row_bytes, "hipMalloc(index scratch)"))) return rc;
+    if ((rc = ensure(ctx, &ctx->d_idx16, &ctx->idx16_bytes, (size_t)n * g.CB * 2, "hipMalloc(idx16 scratch)"))) return rc;
+    if ((rc = hip_check(ctx, hipMemcpyAsync(ctx->d_idx16, idx, (size_t)n * g.CB * 2, hipMemcpyHostToDevice, ctx->stream), "H2D idx"))) return rc;
+    if ((rc = launch_pack_idx(ctx, g, ctx->d_idx16, ctx->d_idx, n))) return rc;
+    if ((rc = launch_gather(ctx, *a, ctx->d_idx, d_out, nullptr, n))) return rc;
+    return finish_output(ctx, g, out, n, out_host);
+}
+
+int pimdl_lutgen(pimdl_ctx* ctx, const float* centroids, const float* weight, uint32_t CB, uint32_t C, uint32_t v,
+                 uint32_t M, uint32_t lut_dtype, uint32_t scale_group, void* lut_out, float* scales_out)
+{
+    if (!ctx) return PIMDL_ERR_INVALID;
+    if (!centroids || !weight || !lut_out) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_lutgen: null argument");
+    if (!CB || !C || !v || !M) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_lutgen: zero-sized dimension");
+    if (lut_dtype != PIMDL_LUT_I8 && lut_dtype != PIMDL_LUT_F32) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_lutgen: unknown lut_dtype");
+    if (lut_dtype == PIMDL_LUT_I8 && !scales_out) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_lutgen: scales_out is null");
+    if (CB > 65535) return set_error(ctx, PIMDL_ERR_UNSUPPORTED, "pimdl_lutgen: more than 65535 codebooks");
+    int rc = activate(ctx);
+    if (rc) return rc;
+    const size_t cent_bytes = (size_t)CB * C * v * 4, w_bytes = (size_t)CB * v * M * 4, lut_elems = (size_t)CB * C * M;
+    const uint32_t ngroups = scale_group ? (CB + scale_group - 1) / scale_group : 1;
+    float *d_cent = nullptr, *d_w = nullptr, *d_lut = nullptr, *d_scales = nullptr;
+    int8_t* d_q = nullptr;
+    rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&d_cent), cent_bytes), "hipMalloc(lutgen centroids)");
+    if (!rc) rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&d_w), w_bytes), "hipMalloc(lutgen weight)");
+    if (!rc) rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&d_lut), lut_elems * 4), "hipMalloc(lutgen lut)");
+    if (!rc) rc = hip_check(ctx, hipMemcpyAsync(d_cent, centroids, cent_bytes, hipMemcpyHostToDevice, ctx->stream), "H2D centroids");
+    if (!rc) rc = hip_check(ctx, hipMemcpyAsync(d_w, weight, w_bytes, hipMemcpyHostToDevice, ctx->stream), "H2D weight");
+    if (!rc) rc = launch_lutgen_f32(ctx, d_cent, d_w, d_lut, CB, C, v, M);
+    if (!rc && lut_dtype == PIMDL_LUT_F32) {
+        rc = hip_check(ctx, hipMemcpyAsync(lut_out, d_lut, lut_elems * 4, hipMemcpyDeviceToHost, ctx->stream), "D2H lut");
+    } else if (!rc) {
+        rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&d_q), lut_elems), "hipMalloc(lutgen q)");
+        if (!rc) rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&d_scales), sizeof(float) * ngroups), "hipMalloc(lutgen scales)");
+        if (!rc) rc = launch_lut_quant(ctx, d_lut, d_q, d_scales, CB, C, M, scale_group);
+        if (!rc) rc = hip_check(ctx, hipMemcpyAsync(lut_out, d_q, lut_elems, hipMemcpyDeviceToHost, ctx->stream), "D2H lut");
+        if (!rc) rc = hip_check(ctx, hipMemcpyAsync(scales_out, d_scales, sizeof(float) * ngroups, hipMemcpyDeviceToHost, ctx->stream), "D2H scales");
+    }
+    if (!rc) rc = hip_check(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+    else (void)hipStreamSynchronize(ctx->stream);
+    (void)hipFree(d_cent);
+    (void)hipFree(d_w);
+    (void)hipFree(d_lut);
+    (void)hipFree(d_q);
+    (void)hipFree(d_scales);
+    return rc;
+}
+
+int pimdl_get_device_info(pimdl_ctx* ctx, pimdl_device_info* info)
+{
+    if (!ctx || !info) return PIMDL_ERR_INVALID;
+    memset(info, 0, sizeof(*info));
+    strncpy(info->name, ctx->prop.name, sizeof(info->name) - 1);
+    strncpy(info->arch, ctx->prop.gcnArchName, sizeof(info->arch) - 1);
+    info->compute_units = ctx->prop.multiProcessorCount;
+    info->clock_khz = ctx->prop.clockRate;
+    info->lds_bytes_per_cu = (uint32_t)ctx->prop.maxSharedMemoryPerMultiProcessor;
+    info->hbm_bytes = ctx->prop.totalGlobalMem;
+    return PIMDL_OK;
+}
+
+int pimdl_amm_get_geometry(const pimdl_amm* a, pimdl_amm_geometry* out)
+{
+    if (!a || !out) return PIMDL_ERR_INVALID;
+    const AmmGeom& g = a->g;
+    out->num_codebook = g.CB;
+    out->num_codebook_padded = g.CB_pad;
+    out->idx_bits = g.idx_bits;
+    out->idx_row_bytes = g.idx_row_bytes;
+    out->col_block = g.col_block;
+    out->row_pitch = g.row_pitch;
+    out->cb_per_slice = g.cb_per_slice;
+    out->lds_bytes = g.gather_lds_bytes;
+    out->tokens_per_wg = g.tokens_per_wg;
+    out->gather_threads = g.gather_threads;
+    out->ccs_tokens_per_wg = 256;
+    out->ccs_cb_per_wg = g.ccs_cb_per_wg;
+    out->ccs_threads = 256;
+    out->ccs_lds_bytes = g.ccs_lds_bytes;
+    return PIMDL_OK;
+}
+
+int pimdl_diag_bandwidth(pimdl_ctx* ctx, uint64_t bytes, float* copy_gbps, float* lds_gbps)
+{
+    if (!ctx) return PIMDL_ERR_INVALID;
+    int rc = activate(ctx);
+    if (rc) return rc;
+    return launch_diag(ctx, bytes, copy_gbps, lds_gbps);
+}
+
+}  // extern "C"

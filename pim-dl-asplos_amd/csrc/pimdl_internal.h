@@ -1,0 +1,91 @@
+// Internal declarations shared by the HIP translation units of libpimdl (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+
+#include "pimdl.h"
+
+namespace pimdl {
+
+// ---------------------------------------------------------------------------------------------
+// Geometry of one AMM operator as the kernels see it.
+//
+// Index rows   [N][idx_row_bytes] bytes; IDX_BITS = 4 (C <= 16, codebook 2k in the low nibble
+//              of byte k) or 8.  Codebooks are padded to a multiple of 32 with index 0.
+// int8 LUT     tiled [M_pad / col_block][CB_pad][C_tile][col_block] bytes (col_block = 16*Q):
+//              one (column block, codebook range) slice is contiguous, so staging it into LDS
+//              is a flat copy.  Padded codebooks / centroid rows / columns hold zeros.
+// fp32 LUT     tiled the same way with col_block floats per row.
+// ---------------------------------------------------------------------------------------------
+struct AmmGeom {
+    uint32_t K, v, CB, CB_pad, C, C_tile, M, M_pad;
+    uint32_t idx_bits, idx_row_bytes;
+    // gather kernel
+    uint32_t q;             // 16-byte chunks per LUT row in LDS
+    uint32_t col_block;     // columns per workgroup (int8: 16*q, fp32: 4*q)
+    uint32_t row_pitch;     // bytes between LUT rows in LDS (16*q + 16: bank-conflict-free b128 gathers)
+    uint32_t gq;            // int8: codebooks per lane group per slice; slice = 4*gq codebooks
+    uint32_t cb_per_slice;
+    uint32_t gather_threads, tokens_per_wg, gather_lds_bytes;
+    // ccs kernel
+    uint32_t ccs_row_floats, ccs_cb_per_wg, ccs_lds_bytes;
+};
+
+struct Ctx;
+
+struct Amm {
+    Ctx* ctx;
+    pimdl_amm_desc desc;
+    AmmGeom g;
+    float* d_centroids;  // [CB][C][v]
+    void* d_lut;         // tiled
+    size_t lut_bytes;
+    float* d_scales;     // int8: scales
+    uint32_t nscales;
+    float* d_bias;       // [M]
+    float h_scale0;
+};
+
+struct Ctx {
+    int device;
+    hipStream_t own_stream;
+    hipStream_t stream;
+    hipDeviceProp_t prop;
+    std::string err;
+    // grow-only device scratch
+    float* d_in;
+    size_t in_bytes;
+    float* d_out;
+    size_t out_bytes;
+    uint8_t* d_idx;
+    size_t idx_bytes;
+    int32_t* d_acc;
+    size_t acc_bytes;
+    uint16_t* d_idx16;
+    size_t idx16_bytes;
+    hipEvent_t ev[4];
+};
+
+int set_error(Ctx* ctx, int code, const char* fmt, ...);
+int hip_check(Ctx* ctx, hipError_t e, const char* what);
+
+// kernels (launchers validate nothing: callers have already checked shapes against AmmGeom)
+int launch_ccs(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_cent, uint8_t* d_idx,
+               uint32_t n);
+int launch_gather(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_t* d_acc_or_null,
+                  uint32_t n);
+int launch_unpack_idx(Ctx* ctx, const AmmGeom& g, const uint8_t* d_idx, uint16_t* d_idx16, uint32_t n,
+                      uint32_t n_stile, uint32_t cb_mtile);
+int launch_pack_idx(Ctx* ctx, const AmmGeom& g, const uint16_t* d_idx16, uint8_t* d_idx, uint32_t n);
+int launch_lutgen_f32(Ctx* ctx, const float* d_cent, const float* d_w, float* d_lut, uint32_t CB,
+                      uint32_t C, uint32_t v, uint32_t M);
+int launch_lut_quant(Ctx* ctx, const float* d_lut, int8_t* d_q, float* d_scales, uint32_t CB, uint32_t C,
+                     uint32_t M, uint32_t scale_group);
+int launch_diag(Ctx* ctx, uint64_t bytes, float* copy_gbps, float* lds_gbps);
+
+uint32_t ccs_cb_per_wg(uint32_t v);  // codebooks one ccs workgroup covers (0: generic kernel)
+bool plan_geometry(const pimdl_amm_desc& d, AmmGeom* g, std::string* why);
+
+}  // namespace pimdl

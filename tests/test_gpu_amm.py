@@ -1,0 +1,207 @@
+"""Parity of the HIP path (through the C ABI) against the CPU oracle, on the same seeded inputs.
+
+Bar: bit-exact centroid indices, bit-exact int32 accumulators, bit-exact fp32 output for the int8
+path (the epilogue is three separately rounded fp32 operations on both sides); fp32-LUT path within
+1e-5 relative (in fact also bit-exact, since both sides add in ascending codebook order)."""
+import numpy as np
+import pytest
+
+import oracle
+from __graft_entry__ import load_package
+
+pimdl = load_package()
+pytestmark = pytest.mark.gpu
+
+THREADS = 8
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = pimdl.Context(0)
+    yield c
+    c.close()
+
+
+def make_case(seed, N, K, v, C, M, lut="i8", dist="normal"):
+    rng = np.random.default_rng(seed)
+    CB = K // v
+    if dist == "normal":
+        x = rng.standard_normal((N, K)).astype(np.float32)
+        cent = rng.standard_normal((CB, C, v)).astype(np.float32)
+    else:  # the reference driver's ranges (test_amm.cpp:26-45)
+        x = rng.uniform(-5, 5, (N, K)).astype(np.float32)
+        cent = rng.uniform(-10, 10, (CB, C, v)).astype(np.float32)
+    bias = rng.standard_normal(M).astype(np.float32)
+    if lut == "i8":
+        table = rng.integers(-128, 128, (CB, C, M)).astype(np.int8)
+    else:
+        table = rng.standard_normal((CB, C, M)).astype(np.float32)
+    return x, cent, table, bias
+
+
+def check_i8(ctx, seed, N, K, v, C, M, scale=0.0123, lut_bias=0.0, bias_mode=0, dist="normal", max_n=None):
+    x, cent, lut, bias = make_case(seed, N, K, v, C, M, "i8", dist)
+    CB = K // v
+    amm = ctx.amm(cent, lut, np.float32(scale), bias, max_n=max_n or N, lut_bias=lut_bias, bias_mode=bias_mode)
+    out, idx, acc = amm.run_debug(x)
+    want_idx = oracle.index_calculation(x, cent, v, threads=THREADS)
+    want_acc = oracle.gather_i8(want_idx, lut, threads=THREADS)
+    want_out = oracle.dequant(want_acc, bias, CB, scale, lut_bias, bias_mode, threads=THREADS)
+    assert np.array_equal(idx, want_idx), f"indices: {(idx != want_idx).sum()} of {idx.size} differ"
+    assert np.array_equal(acc, want_acc), f"accumulators: {(acc != want_acc).sum()} of {acc.size} differ"
+    assert np.array_equal(out.view(np.uint32), want_out.view(np.uint32)), "fp32 output bits differ"
+    # the plain entry point gives the same bytes as the debug one
+    assert np.array_equal(amm.run(x).view(np.uint32), out.view(np.uint32))
+    amm.close()
+
+
+def test_config1_single_amm(ctx):
+    """N=128, K=768, v=2 (384 codebooks), 16 centroids, M=768, LUT = quantised centroid x W."""
+    rng = np.random.default_rng(0)
+    N, K, v, C, M = 128, 768, 2, 16, 768
+    CB = K // v
+    x = rng.standard_normal((N, K)).astype(np.float32)
+    cent = rng.standard_normal((CB, C, v)).astype(np.float32)
+    W = (rng.standard_normal((K, M)) * 0.02).astype(np.float32)
+    lut, scales = oracle.lut_quant(oracle.lutgen_f32(cent, W, threads=THREADS))
+    bias = np.zeros(M, np.float32)
+    want_out, want_idx, want_acc = oracle.amm_cpu(x, cent, lut, bias, v, float(scales[0]), 0.0, threads=THREADS)
+    amm = ctx.amm(cent, lut, scales, bias, max_n=N)
+    out, idx, acc = amm.run_debug(x)
+    assert np.array_equal(idx, want_idx)
+    assert np.array_equal(acc, want_acc)
+    assert np.array_equal(out.view(np.uint32), want_out.view(np.uint32))
+    amm.close()
+
+
+@pytest.mark.parametrize("v,C", [(2, 8), (2, 16), (2, 32), (4, 8), (4, 16), (4, 32), (8, 8), (8, 16), (8, 32),
+                                 (16, 16), (32, 16), (4, 64), (4, 128), (2, 256)])
+def test_sweep_sub_vector_length_and_centroids(ctx, v, C):
+    check_i8(ctx, 100 + v * 7 + C, N=300, K=64 * v if v < 16 else 96 * v // 2, v=v, C=C, M=200)
+
+
+@pytest.mark.parametrize("N,K,v,C,M", [
+    (1, 8, 4, 16, 4),        # smallest sensible shape
+    (17, 24, 4, 16, 20),     # CB=6 (padded to 32), M not a multiple of the column block
+    (255, 36, 4, 16, 63),    # M % 4 != 0: scalar stores
+    (257, 40, 4, 5, 130),    # C not a power of two
+    (513, 12, 3, 7, 33),     # sub_vec_len with no specialised kernel
+    (64, 10, 5, 20, 18),     # generic v, 8-bit indices, K % 4 != 0
+    (100, 6, 2, 16, 64),     # CB=3 (odd), K % 4 != 0: scalar activation loads
+])
+def test_ragged_shapes(ctx, N, K, v, C, M):
+    check_i8(ctx, N + K + M, N, K, v, C, M)
+
+
+def test_reference_driver_value_ranges_and_bias_modes(ctx):
+    # uniform(-5,5) activations, uniform(-10,10) centroids, scale 0.1, bias 0.2 as in the shipped YAML
+    check_i8(ctx, 7, 256, 128, 4, 16, 96, scale=0.1, lut_bias=0.2, bias_mode=0, dist="uniform")
+    check_i8(ctx, 8, 256, 128, 4, 16, 96, scale=0.1, lut_bias=0.2, bias_mode=1, dist="uniform")
+
+
+def test_golden_reference_vectors_on_gpu(ctx, golden_index):
+    """The fixtures produced by the reference's own compiled index_calculation."""
+    for i in range(int(golden_index["ncases"])):
+        x, cent, want = golden_index[f"c{i}_x"], golden_index[f"c{i}_cent"], golden_index[f"c{i}_idx"]
+        CB, C, v = cent.shape
+        lut = np.zeros((CB, C, 4), np.int8)
+        amm = ctx.amm(cent, lut, np.float32(1.0), None, max_n=x.shape[0])
+        got = amm.index_calculation(x)
+        assert np.array_equal(got, want), f"golden case {i} ({golden_index[f'c{i}_kind']})"
+        for key in golden_index.files:
+            if key.startswith(f"c{i}_tiled_"):
+                _, _, ns, cm = key.split("_")
+                assert np.array_equal(amm.index_calculation(x, int(ns), int(cm)), golden_index[key]), key
+        amm.close()
+
+
+def test_near_ties_follow_the_scan_not_the_true_argmin(ctx):
+    """Inputs midway between two centroids: many distance pairs differ by ~1e-6."""
+    rng = np.random.default_rng(5)
+    N, CB, C, v = 2048, 32, 16, 4
+    cent = rng.standard_normal((CB, C, v)).astype(np.float32)
+    a = rng.integers(0, C, (N, CB))
+    b = (a + 1 + rng.integers(0, C - 1, (N, CB))) % C
+    cb = np.arange(CB)[None, :]
+    mid = (cent[cb, a] + cent[cb, b]) * np.float32(0.5)
+    x = (mid + rng.standard_normal((N, CB, v)).astype(np.float32) * np.float32(2e-7)).reshape(N, CB * v)
+    want = oracle.index_calculation(x, cent, v, threads=THREADS)
+    true_argmin = oracle.np_distances(x, cent).argmin(-1)
+    assert (want != true_argmin).sum() > 100  # the case really separates the two rules
+    amm = ctx.amm(cent, np.zeros((CB, C, 4), np.int8), np.float32(1.0), None, max_n=N)
+    assert np.array_equal(amm.index_calculation(x), want)
+    amm.close()
+
+
+def test_gather_from_given_indices_and_invariants(ctx):
+    rng = np.random.default_rng(21)
+    N, CB, C, M, v = 300, 40, 16, 192, 4
+    cent = rng.standard_normal((CB, C, v)).astype(np.float32)
+    lut = rng.integers(-128, 128, (CB, C, M)).astype(np.int8)
+    idx = rng.integers(0, C, (N, CB)).astype(np.uint16)
+    amm = ctx.amm(cent, lut, np.float32(1.0), None, max_n=N)
+    out = amm.lut_gather(idx)
+    want = oracle.gather_i8(idx, lut, threads=THREADS)
+    assert np.array_equal(out, want.astype(np.float32))
+    amm.close()
+    # extremes: every entry -128 / +127, CB = 768 (the largest of the BERT shapes)
+    CB = 768
+    cent = rng.standard_normal((CB, C, v)).astype(np.float32)
+    idx = rng.integers(0, C, (64, CB)).astype(np.uint16)
+    for val in (-128, 127):
+        amm = ctx.amm(cent, np.full((CB, C, 64), val, np.int8), np.float32(1.0), None, max_n=64)
+        assert (amm.lut_gather(idx) == float(val * CB)).all()
+        amm.close()
+
+
+@pytest.mark.parametrize("C,v", [(16, 4), (8, 2), (32, 8)])
+def test_fp32_lut_path(ctx, C, v):
+    N, K, M = 300, 48 * v, 100
+    x, cent, lut, bias = make_case(31 + C, N, K, v, C, M, "f32")
+    amm = ctx.amm(cent, lut, None, bias, max_n=N)
+    out, idx, _ = amm.run_debug(x)
+    want_idx = oracle.index_calculation(x, cent, v, threads=THREADS)
+    assert np.array_equal(idx, want_idx)
+    want = oracle.gather_f32(want_idx, lut, bias, threads=THREADS)
+    np.testing.assert_allclose(out, want, rtol=1e-5, atol=1e-6)  # the stated tolerance for fp32 paths
+    amm.close()
+
+
+def test_device_pointers_and_partial_batches(ctx):
+    """Inputs already resident in HBM (torch tensors), n smaller than max_n, output rows past n untouched."""
+    import torch
+
+    N, K, v, C, M = 700, 256, 4, 16, 320
+    x, cent, lut, bias = make_case(41, N, K, v, C, M)
+    amm = ctx.amm(cent, lut, np.float32(0.05), bias, max_n=1024)
+    want = oracle.amm_cpu(x, cent, lut, bias, v, 0.05, 0.0, threads=THREADS)[0]
+    xd = torch.from_numpy(x).cuda()
+    od = torch.full((1024, M), -7.0, device="cuda")
+    torch.cuda.synchronize()
+    amm.run_ptr(xd.data_ptr(), N, od.data_ptr())
+    ctx.synchronize()
+    got = od.cpu().numpy()
+    assert np.array_equal(got[:N].view(np.uint32), want.view(np.uint32))
+    assert (got[N:] == -7.0).all()
+    # a second, smaller batch through the same operator
+    amm.run_ptr(xd.data_ptr(), 33, od.data_ptr())
+    ctx.synchronize()
+    assert np.array_equal(od.cpu().numpy()[:33].view(np.uint32), want[:33].view(np.uint32))
+    amm.close()
+
+
+def test_error_paths(ctx):
+    cent = np.zeros((4, 16, 4), np.float32)
+    lut = np.zeros((4, 16, 8), np.int8)
+    with pytest.raises(pimdl.PimdlError) as e:
+        ctx.amm(cent, lut, None, None)           # int8 LUT without scales
+    assert e.value.code == -1
+    with pytest.raises(pimdl.PimdlError) as e:
+        ctx.amm(cent, lut, np.float32(1), None, scale_group=3)
+    assert e.value.code == -2
+    amm = ctx.amm(cent, lut, np.float32(1), None, max_n=8)
+    with pytest.raises(pimdl.PimdlError) as e:
+        amm.run(np.zeros((9, 16), np.float32))   # n > max_n
+    assert e.value.code == -1
+    assert amm.run(np.zeros((0, 16), np.float32)).shape == (0, 8)  # empty batch is a no-op
+    amm.close()
