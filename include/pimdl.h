@@ -130,15 +130,41 @@ PIMDL_API int pimdl_amm_profile(pimdl_amm* amm, const float* in_dev, uint32_t n,
 
 /* ---- the two halves on their own ---------------------------------------------------------
  * pimdl_index_calculation replaces index_calculation (src/host/index_calc_host.h:5,
- * index_calc_host.cpp:8-53).  in is host or device fp32 [n][K]; idx_out is HOST uint16, written
- * at the reference's tiled offset (index_calc_host.cpp:41-49); n_stile_size == n and
- * cb_mtile_size == CB give row-major [n][CB].  Uses the operator's resident centroids. */
-PIMDL_API int pimdl_index_calculation(pimdl_amm* amm, const float* in, uint32_t n,
-                                      uint16_t* idx_out, uint32_t n_stile_size,
-                                      uint32_t cb_mtile_size);
+ * index_calc_host.cpp:8-53) with its own argument list: in is host or device fp32 [n][K],
+ * centroids is HOST fp32 [K/v][C][v] (uploaded on every call, as the reference reads it on every
+ * call), idx_out is HOST uint16, written at the reference's tiled offset
+ * (index_calc_host.cpp:41-49); n_stile_size == n and cb_mtile_size == K/v give row-major. */
+PIMDL_API int pimdl_index_calculation(pimdl_ctx* ctx, const float* in, const float* centroids,
+                                      uint32_t n, uint32_t input_feature_len, uint32_t sub_vec_len,
+                                      uint32_t num_centroid, uint16_t* idx_out,
+                                      uint32_t n_stile_size, uint32_t cb_mtile_size);
+/* The same with an operator's resident centroids (no upload). */
+PIMDL_API int pimdl_amm_index_calculation(pimdl_amm* amm, const float* in, uint32_t n,
+                                          uint16_t* idx_out, uint32_t n_stile_size,
+                                          uint32_t cb_mtile_size);
 /* pimdl_lut_gather replaces pim_lut (src/host/pim_lut_host.h:13-14, pim_lut_host.cpp:121-222):
  * idx is HOST uint16 row-major [n][CB] holding centroid ids; out is host or device fp32 [n][M]. */
 PIMDL_API int pimdl_lut_gather(pimdl_amm* amm, const uint16_t* idx, uint32_t n, float* out);
+
+/* ---- the reference's DPU tile orders ---------------------------------------------------------
+ * The reference's amm_host / pim_lut hand back the output in the order the DPUs produced it, and
+ * pim_lut takes the index buffer in the order index_calculation wrote it.  These variants keep
+ * those orders so the C++ layer with the reference's signatures can sit on this ABI.
+ *   index offset  (n / ns)*ns*CB + (cb / cm)*ns*cm + (n % ns)*cm + cb % cm
+ *                 ns = n_stile_size, cm = cb_mtile_size          (index_calc_host.cpp:41-49)
+ *   output offset dpu*ns*fs + ((f % fs) / fm)*ns*fm + (n % ns)*fm + (f % fs) % fm,
+ *                 dpu = (n / ns)*(M / fs) + f / fs, fs = feature_stile_size,
+ *                 fm = feature_mtile_size                         (test/test_amm.cpp:193-202)
+ * A zero field means "identity" (ns = n, cm = CB, fs = fm = M), i.e. row-major. */
+typedef struct pimdl_tiling {
+    uint32_t n_stile_size, cb_mtile_size, feature_stile_size, feature_mtile_size;
+} pimdl_tiling;
+/* amm_host with the reference's output order.  in host or device; out host or device. */
+PIMDL_API int pimdl_amm_run_tiled(pimdl_amm* amm, const float* in, uint32_t n, float* out,
+                                  const pimdl_tiling* tiling);
+/* pim_lut with the reference's index and output orders.  idx is HOST uint16 centroid ids. */
+PIMDL_API int pimdl_lut_gather_tiled(pimdl_amm* amm, const uint16_t* idx, uint32_t n, float* out,
+                                     const pimdl_tiling* tiling);
 
 /* ---- LUT construction ----------------------------------------------------------------------
  * Replaces model-calibration/pim_weight_converter.py:82-91 (bmm of centroids with the weight)

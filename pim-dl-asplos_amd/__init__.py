@@ -25,7 +25,8 @@ STATUS = {0: "PIMDL_OK", -1: "PIMDL_ERR_INVALID", -2: "PIMDL_ERR_UNSUPPORTED", -
 # every symbol include/pimdl.h declares
 EXPORTS = ["pimdl_init", "pimdl_destroy", "pimdl_last_error", "pimdl_set_stream", "pimdl_synchronize",
            "pimdl_amm_create", "pimdl_amm_destroy", "pimdl_amm_run", "pimdl_amm_run_debug",
-           "pimdl_amm_profile", "pimdl_index_calculation", "pimdl_lut_gather", "pimdl_lutgen",
+           "pimdl_amm_profile", "pimdl_index_calculation", "pimdl_amm_index_calculation", "pimdl_lut_gather",
+           "pimdl_amm_run_tiled", "pimdl_lut_gather_tiled", "pimdl_lutgen",
            "pimdl_get_device_info", "pimdl_amm_get_geometry", "pimdl_diag_bandwidth"]
 
 
@@ -51,6 +52,11 @@ class DeviceInfo(ctypes.Structure):
     _fields_ = [("name", ctypes.c_char * 64), ("arch", ctypes.c_char * 32),
                 ("compute_units", ctypes.c_uint32), ("clock_khz", ctypes.c_uint32),
                 ("lds_bytes_per_cu", ctypes.c_uint32), ("hbm_bytes", ctypes.c_uint64)]
+
+
+class Tiling(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_uint32) for n in ("n_stile_size", "cb_mtile_size", "feature_stile_size",
+                                               "feature_mtile_size")]
 
 
 class AmmGeometry(ctypes.Structure):
@@ -107,7 +113,10 @@ def lib():
     L.pimdl_amm_run.argtypes = [vp, vp, u32, vp]
     L.pimdl_amm_run_debug.argtypes = [vp, vp, u32, vp, vp, vp]
     L.pimdl_amm_profile.argtypes = [vp, vp, u32, vp, u32, u32, ctypes.POINTER(AmmTiming)]
-    L.pimdl_index_calculation.argtypes = [vp, vp, u32, vp, u32, u32]
+    L.pimdl_index_calculation.argtypes = [vp, vp, vp, u32, u32, u32, u32, vp, u32, u32]
+    L.pimdl_amm_index_calculation.argtypes = [vp, vp, u32, vp, u32, u32]
+    L.pimdl_amm_run_tiled.argtypes = [vp, vp, u32, vp, ctypes.POINTER(Tiling)]
+    L.pimdl_lut_gather_tiled.argtypes = [vp, vp, u32, vp, ctypes.POINTER(Tiling)]
     L.pimdl_lut_gather.argtypes = [vp, vp, u32, vp]
     L.pimdl_lutgen.argtypes = [vp, vp, vp, u32, u32, u32, u32, u32, u32, vp, vp]
     L.pimdl_get_device_info.argtypes = [vp, ctypes.POINTER(DeviceInfo)]
@@ -170,6 +179,17 @@ class Context:
         self._check(lib().pimdl_diag_bandwidth(self._h, nbytes, ctypes.byref(c) if copy else None,
                                                ctypes.byref(l) if lds else None))
         return c.value, l.value
+
+    def index_calculation(self, x, centroids, n_stile=0, cb_mtile=0):
+        """Context-level closest-centroid search: centroids are passed (and uploaded) per call."""
+        x = np.ascontiguousarray(x, np.float32)
+        centroids = np.ascontiguousarray(centroids, np.float32)
+        n, K = x.shape
+        CB, C, v = centroids.shape
+        idx = np.empty(n * CB, np.uint16)
+        self._check(lib().pimdl_index_calculation(self._h, _ptr(x), _ptr(centroids), n, K, v, C, _ptr(idx), n_stile,
+                                                  cb_mtile))
+        return idx.reshape(n, CB) if (n_stile in (0, n) and cb_mtile in (0, CB)) else idx
 
     def lutgen(self, centroids, weight, lut_dtype=LUT_I8, scale_group=0):
         """centroids f32 [CB][C][v], weight f32 [K][M] -> (lut [CB][C][M], scales or None)."""
@@ -264,8 +284,24 @@ class Amm:
         n_stile = n if n_stile is None else n_stile
         cb_mtile = self.CB if cb_mtile is None else cb_mtile
         idx = np.empty(n * self.CB, np.uint16)
-        self.ctx._check(lib().pimdl_index_calculation(self._h, _ptr(x), n, _ptr(idx), n_stile, cb_mtile))
+        self.ctx._check(lib().pimdl_amm_index_calculation(self._h, _ptr(x), n, _ptr(idx), n_stile, cb_mtile))
         return idx.reshape(n, self.CB) if (n_stile == n and cb_mtile == self.CB) else idx
+
+    def run_tiled(self, x, n_stile=0, cb_mtile=0, f_stile=0, f_mtile=0):
+        """Output as a flat array in the reference's DPU order (test_amm.cpp:193-202)."""
+        x = np.ascontiguousarray(x, np.float32)
+        n = x.shape[0]
+        out = np.empty(n * self.M, np.float32)
+        til = Tiling(n_stile, cb_mtile, f_stile, f_mtile)
+        self.ctx._check(lib().pimdl_amm_run_tiled(self._h, _ptr(x), n, _ptr(out), ctypes.byref(til)))
+        return out
+
+    def lut_gather_tiled(self, idx_flat, n, n_stile=0, cb_mtile=0, f_stile=0, f_mtile=0):
+        idx_flat = np.ascontiguousarray(idx_flat, np.uint16).reshape(-1)
+        out = np.empty(n * self.M, np.float32)
+        til = Tiling(n_stile, cb_mtile, f_stile, f_mtile)
+        self.ctx._check(lib().pimdl_lut_gather_tiled(self._h, _ptr(idx_flat), n, _ptr(out), ctypes.byref(til)))
+        return out
 
     def lut_gather(self, idx):
         idx = np.ascontiguousarray(idx, np.uint16)

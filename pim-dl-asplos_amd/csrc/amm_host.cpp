@@ -1,0 +1,248 @@
+// C++ host layer with the reference's operator API (include/pimdl/amm_host.h) on top of the C ABI.
+// Plain host code: everything that touches the GPU goes through include/pimdl.h.
+#include "pimdl/amm_host.h"
+
+#include <string.h>
+
+#include <map>
+#include <mutex>
+#include <stdexcept>
+#include <tuple>
+#include <vector>
+
+#include "pimdl.h"
+
+#define PIMDL_HOST_API __attribute__((visibility("default")))
+
+namespace {
+
+struct Cached {
+    pimdl_amm* amm;
+    uint64_t fingerprint;
+    uint32_t max_n;
+};
+
+// key: lut pointer, centroid pointer, bias pointer, N-independent shape, layout, scale, bias
+typedef std::tuple<const void*, const void*, const void*, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t,
+                   uint32_t>
+    Key;
+
+std::mutex g_mu;
+std::map<std::pair<pimdl_ctx*, Key>, Cached> g_cache;
+pimdl_ctx* g_implicit_ctx = nullptr;
+PimdlHostOptions g_opts;
+
+[[noreturn]] void fail(pimdl_ctx* ctx, const char* what)
+{
+    throw std::runtime_error(std::string(what) + ": " + pimdl_last_error(ctx));
+}
+
+pimdl_ctx* ctx_of(dpu_set_t* s)
+{
+    if (!s || !s->impl) throw std::runtime_error("dpu_set_t is not allocated (call allocate_dpu / allocate_rank first)");
+    return static_cast<pimdl_ctx*>(s->impl);
+}
+
+pimdl_ctx* implicit_ctx()
+{
+    if (!g_implicit_ctx && pimdl_init(g_opts.device, &g_implicit_ctx)) fail(nullptr, "pimdl_init");
+    return g_implicit_ctx;
+}
+
+// every 4 KiB one 8-byte word, plus the last word: cheap, catches wholesale replacement of a LUT
+uint64_t fingerprint(const void* p, size_t bytes)
+{
+    const unsigned char* b = static_cast<const unsigned char*>(p);
+    uint64_t h = 1469598103934665603ull ^ bytes;
+    for (size_t off = 0; off + 8 <= bytes; off += 4096) {
+        uint64_t w;
+        memcpy(&w, b + off, 8);
+        h = (h ^ w) * 1099511628211ull;
+    }
+    if (bytes >= 8) {
+        uint64_t w;
+        memcpy(&w, b + bytes - 8, 8);
+        h = (h ^ w) * 1099511628211ull;
+    }
+    return h;
+}
+
+uint32_t lut_tile(const LUTParams& lp)
+{
+    return lp.lut_load_type == STATIC ? lp.feature_stile_size : lp.feature_load_tile_size;
+}
+
+// [f_tile][cb][c][f_in_tile] (test_amm.cpp:82-92,106-116) -> canonical [cb][c][M]
+void untile_lut(const lut_data_type* dpu_lut, lut_data_type* canon, uint32_t CB, uint32_t C, uint32_t M, uint32_t ft)
+{
+    const uint32_t ntile = M / ft;
+    for (uint32_t t = 0; t < ntile; ++t)
+        for (uint32_t cb = 0; cb < CB; ++cb)
+            for (uint32_t c = 0; c < C; ++c)
+                memcpy(canon + ((size_t)cb * C + c) * M + (size_t)t * ft,
+                       dpu_lut + (size_t)t * CB * C * ft + ((size_t)cb * C + c) * ft, ft);
+}
+
+pimdl_amm* get_operator(pimdl_ctx* ctx, const float* centroids, uint32_t K, uint32_t v, const lut_data_type* lut,
+                        const float* bias, const LUTParams& lp)
+{
+    const uint32_t CB = lp.num_codebook, C = lp.num_centroid, M = lp.output_feature_len;
+    uint32_t ft = lut_tile(lp);
+    if (ft == 0 || ft > M) ft = M;
+    if (M % ft) throw std::runtime_error("LUT feature tile does not divide output_feature_len");
+    uint32_t scale_bits, bias_bits;
+    memcpy(&scale_bits, &lp.scale, 4);
+    memcpy(&bias_bits, &lp.bias, 4);
+    const Key key(lut, centroids, bias, K, v, C, M, ft, scale_bits, bias_bits);
+    const size_t lut_bytes = (size_t)CB * C * M;
+    const uint64_t fp = fingerprint(lut, lut_bytes) ^ (centroids ? fingerprint(centroids, (size_t)CB * C * v * 4) : 0);
+
+    std::lock_guard<std::mutex> lock(g_mu);
+    auto it = g_cache.find(std::make_pair(ctx, key));
+    if (it != g_cache.end()) {
+        if (it->second.fingerprint == fp && it->second.max_n >= lp.n) return it->second.amm;
+        pimdl_amm_destroy(it->second.amm);
+        g_cache.erase(it);
+    }
+    std::vector<lut_data_type> canon;
+    const lut_data_type* canon_ptr = lut;
+    if (ft != M) {
+        canon.resize(lut_bytes);
+        untile_lut(lut, canon.data(), CB, C, M, ft);
+        canon_ptr = canon.data();
+    }
+    std::vector<float> dummy_centroids;
+    if (!centroids) {  // pim_lut() alone never searches centroids
+        dummy_centroids.assign((size_t)CB * C * v, 0.0f);
+        centroids = dummy_centroids.data();
+    }
+    pimdl_amm_desc d;
+    memset(&d, 0, sizeof(d));
+    d.max_n = lp.n;
+    d.input_feature_len = K;
+    d.sub_vec_len = v;
+    d.num_centroid = C;
+    d.output_feature_len = M;
+    d.lut_dtype = PIMDL_LUT_I8;
+    d.scale_group = 0;
+    d.bias_mode = PIMDL_BIAS_TIMES_CB;  // pim_lut_host.cpp:201
+    d.lut_bias = lp.bias;
+    pimdl_amm* amm = nullptr;
+    if (pimdl_amm_create(ctx, &d, centroids, canon_ptr, &lp.scale, bias, &amm)) fail(ctx, "pimdl_amm_create");
+    g_cache[std::make_pair(ctx, key)] = Cached{amm, fp, lp.n};
+    return amm;
+}
+
+pimdl_tiling tiling_of(const LUTParams& lp)
+{
+    pimdl_tiling t;
+    t.n_stile_size = lp.n_stile_size;
+    t.cb_mtile_size = lp.cb_mtile_size;
+    t.feature_stile_size = lp.feature_stile_size;
+    t.feature_mtile_size = lp.feature_mtile_size;
+    return t;
+}
+
+// pim_lut_host.cpp:40-104: the in-place rewrite of centroid ids into DPU table offsets
+void mutate_index(const LUTParams& lp, index_data_type* idx)
+{
+    const uint32_t ns = lp.n_stile_size ? lp.n_stile_size : lp.n;
+    const uint32_t cm = lp.cb_mtile_size ? lp.cb_mtile_size : lp.num_codebook;
+    for (uint32_t n = 0; n < lp.n; ++n)
+        for (uint32_t cb = 0; cb < lp.num_codebook; ++cb) {
+            const uint32_t ci = cb % cm;
+            const size_t off = (size_t)(n / ns) * ns * lp.num_codebook + (size_t)(cb / cm) * ns * cm +
+                               (size_t)(n % ns) * cm + ci;
+            if (lp.lut_load_type == STATIC)
+                idx[off] = (index_data_type)(idx[off] * lp.feature_stile_size);
+            else if (lp.lut_load_type == FINE_GRAIN)
+                idx[off] = (index_data_type)(idx[off] * lp.feature_load_tile_size);
+            else
+                idx[off] = (index_data_type)((ci % lp.cb_load_tile_size) * lp.num_centroid * lp.feature_load_tile_size +
+                                             idx[off] * lp.feature_load_tile_size);
+        }
+}
+
+}  // namespace
+
+PIMDL_HOST_API PimdlHostOptions& pimdl_host_options() { return g_opts; }
+
+PIMDL_HOST_API void pimdl_host_invalidate(const void* lut_table)
+{
+    std::lock_guard<std::mutex> lock(g_mu);
+    for (auto it = g_cache.begin(); it != g_cache.end();) {
+        if (std::get<0>(it->first.second) == lut_table) {
+            pimdl_amm_destroy(it->second.amm);
+            it = g_cache.erase(it);
+        } else {
+            ++it;
+        }
+    }
+}
+
+PIMDL_HOST_API uint32_t allocate_dpu(dpu_set_t* dpu_set, uint32_t dpu_num)
+{
+    pimdl_ctx* ctx = nullptr;
+    if (pimdl_init(g_opts.device, &ctx)) fail(nullptr, "allocate_dpu: pimdl_init");
+    dpu_set->impl = ctx;
+    return dpu_num;
+}
+
+PIMDL_HOST_API uint32_t allocate_rank(dpu_set_t* dpu_set, uint32_t rank_num)
+{
+    allocate_dpu(dpu_set, rank_num * 64);
+    return rank_num * 64;  // NR_DPUS_PER_RANK
+}
+
+PIMDL_HOST_API void free_dpu_set(dpu_set_t* dpu_set)
+{
+    if (!dpu_set || !dpu_set->impl) return;
+    pimdl_ctx* ctx = static_cast<pimdl_ctx*>(dpu_set->impl);
+    {
+        std::lock_guard<std::mutex> lock(g_mu);
+        for (auto it = g_cache.begin(); it != g_cache.end();) {
+            if (it->first.first == ctx) {
+                pimdl_amm_destroy(it->second.amm);
+                it = g_cache.erase(it);
+            } else {
+                ++it;
+            }
+        }
+    }
+    pimdl_destroy(ctx);
+    dpu_set->impl = nullptr;
+}
+
+PIMDL_HOST_API void load_binary(dpu_set_t*, std::string) {}  // the kernels live in the library
+
+PIMDL_HOST_API void index_calculation(float* input_tensor, float* centroid_tensor, index_data_type* lut_input_index,
+                                      IndexCalcParams p)
+{
+    pimdl_ctx* ctx = implicit_ctx();
+    if (pimdl_index_calculation(ctx, input_tensor, centroid_tensor, p.n, p.input_feature_len, p.sub_vec_len,
+                                p.num_centroid, lut_input_index, p.n_stile_size, p.cb_mtile_size))
+        fail(ctx, "index_calculation");
+}
+
+PIMDL_HOST_API void pim_lut(LUTParams lp, dpu_set_t* dpu_set, index_data_type* input_index, lut_data_type* lut_table,
+                            float* bias_tensor, float* output_tensor)
+{
+    pimdl_ctx* ctx = ctx_of(dpu_set);
+    // K and v are irrelevant to the gather; the operator is keyed with v = 1, K = num_codebook
+    pimdl_amm* amm = get_operator(ctx, nullptr, lp.num_codebook, 1, lut_table, bias_tensor, lp);
+    const pimdl_tiling t = tiling_of(lp);
+    if (pimdl_lut_gather_tiled(amm, input_index, lp.n, output_tensor, &t)) fail(ctx, "pim_lut");
+    if (g_opts.mutate_index_buffer) mutate_index(lp, input_index);
+}
+
+PIMDL_HOST_API void amm_host(dpu_set_t* dpu_set, float* input_tensor, float* centroid_tensor, lut_data_type* lut_table,
+                             float* bias_tensor, float* output_tensor, IndexCalcParams ip, LUTParams lp)
+{
+    pimdl_ctx* ctx = ctx_of(dpu_set);
+    if (ip.n != lp.n || ip.num_codebook != lp.num_codebook || ip.num_centroid != lp.num_centroid ||
+        ip.input_feature_len != ip.num_codebook * ip.sub_vec_len)
+        throw std::runtime_error("amm_host: index_params and lut_params disagree");
+    pimdl_amm* amm = get_operator(ctx, centroid_tensor, ip.input_feature_len, ip.sub_vec_len, lut_table, bias_tensor, lp);
+    const pimdl_tiling t = tiling_of(lp);
+    if (pimdl_amm_run_tiled(amm, input_tensor, lp.n, output_tensor, &t)) fail(ctx, "amm_host");
+}

@@ -193,10 +193,10 @@ __global__ void unpack_idx_kernel(const uint8_t* __restrict__ idx, uint16_t* __r
     out[off] = val;
 }
 
-// row-major uint16 [N][CB] -> packed rows (padded codebooks get index 0)
+// uint16 centroid ids at the reference's tiled offset -> packed rows (padded codebooks get index 0)
 template <int IDX_BITS>
 __global__ void pack_idx_kernel(const uint16_t* __restrict__ in, uint8_t* __restrict__ idx, uint32_t N,
-                                uint32_t CB, uint32_t idx_row_bytes)
+                                uint32_t CB, uint32_t idx_row_bytes, uint32_t n_stile, uint32_t cb_mtile)
 {
     constexpr int CB_PER_BYTE = 8 / IDX_BITS;
     const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -205,7 +205,11 @@ __global__ void pack_idx_kernel(const uint16_t* __restrict__ in, uint8_t* __rest
     uint32_t outv = 0;
     for (int h = 0; h < CB_PER_BYTE; ++h) {
         const uint32_t cb = byte * CB_PER_BYTE + h;
-        if (cb < CB) outv |= (uint32_t)(in[(size_t)n * CB + cb] & ((1u << IDX_BITS) - 1)) << (IDX_BITS * h);
+        if (cb < CB) {
+            const uint64_t off = (uint64_t)(n / n_stile) * n_stile * CB + (uint64_t)(cb / cb_mtile) * n_stile * cb_mtile +
+                                 (uint64_t)(n % n_stile) * cb_mtile + (cb % cb_mtile);
+            outv |= (uint32_t)(in[off] & ((1u << IDX_BITS) - 1)) << (IDX_BITS * h);
+        }
     }
     idx[gid] = (uint8_t)outv;
 }
@@ -276,18 +280,45 @@ int launch_unpack_idx(Ctx* ctx, const AmmGeom& g, const uint8_t* d_idx, uint16_t
     return hip_check(ctx, hipGetLastError(), "unpack_idx_kernel launch");
 }
 
-int launch_pack_idx(Ctx* ctx, const AmmGeom& g, const uint16_t* d_idx16, uint8_t* d_idx, uint32_t n)
+int launch_pack_idx(Ctx* ctx, const AmmGeom& g, const uint16_t* d_idx16, uint8_t* d_idx, uint32_t n,
+                    uint32_t n_stile, uint32_t cb_mtile)
 {
     if (n == 0) return PIMDL_OK;
     const uint64_t total = (uint64_t)n * g.idx_row_bytes;
     dim3 grid((uint32_t)((total + 255) / 256));
     if (g.idx_bits == 4)
         hipLaunchKernelGGL((pack_idx_kernel<4>), grid, dim3(256), 0, ctx->stream, d_idx16, d_idx, n, g.CB,
-                           g.idx_row_bytes);
+                           g.idx_row_bytes, n_stile, cb_mtile);
     else
         hipLaunchKernelGGL((pack_idx_kernel<8>), grid, dim3(256), 0, ctx->stream, d_idx16, d_idx, n, g.CB,
-                           g.idx_row_bytes);
+                           g.idx_row_bytes, n_stile, cb_mtile);
     return hip_check(ctx, hipGetLastError(), "pack_idx_kernel launch");
+}
+
+namespace {
+// row-major [N][M] -> the order the reference's DPUs hand the output back in (test_amm.cpp:193-202)
+__global__ void retile_output_kernel(const float* __restrict__ in, float* __restrict__ out, uint32_t N, uint32_t M,
+                                     uint32_t n_stile, uint32_t f_stile, uint32_t f_mtile)
+{
+    const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= (uint64_t)N * M) return;
+    const uint32_t n = gid / M, f = gid % M;
+    const uint64_t dpu = (uint64_t)(n / n_stile) * (M / f_stile) + f / f_stile;
+    const uint32_t row = n % n_stile, dim = f % f_stile;
+    const uint64_t off = dpu * n_stile * f_stile + (uint64_t)(dim / f_mtile) * n_stile * f_mtile +
+                         (uint64_t)row * f_mtile + dim % f_mtile;
+    out[off] = in[gid];
+}
+}  // namespace
+
+int launch_retile_output(Ctx* ctx, const float* d_rowmajor, float* d_tiled, uint32_t n, uint32_t M, uint32_t n_stile,
+                         uint32_t f_stile, uint32_t f_mtile)
+{
+    if (n == 0) return PIMDL_OK;
+    const uint64_t total = (uint64_t)n * M;
+    hipLaunchKernelGGL(retile_output_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, ctx->stream,
+                       d_rowmajor, d_tiled, n, M, n_stile, f_stile, f_mtile);
+    return hip_check(ctx, hipGetLastError(), "retile_output_kernel launch");
 }
 
 }  // namespace pimdl

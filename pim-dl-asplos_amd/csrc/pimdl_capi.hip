@@ -163,6 +163,8 @@ int pimdl_init(int device, pimdl_ctx** out)
     ctx->d_idx = nullptr; ctx->idx_bytes = 0;
     ctx->d_acc = nullptr; ctx->acc_bytes = 0;
     ctx->d_idx16 = nullptr; ctx->idx16_bytes = 0;
+    ctx->d_tmp = nullptr; ctx->tmp_bytes = 0;
+    ctx->d_cent = nullptr; ctx->cent_bytes = 0;
     for (auto& ev : ctx->ev) ev = nullptr;
     int rc = hip_check(ctx, hipSetDevice(device), "hipSetDevice");
     if (!rc) rc = hip_check(ctx, hipGetDeviceProperties(&ctx->prop, device), "hipGetDeviceProperties");
@@ -192,6 +194,8 @@ int pimdl_destroy(pimdl_ctx* ctx)
     (void)hipFree(ctx->d_idx);
     (void)hipFree(ctx->d_acc);
     (void)hipFree(ctx->d_idx16);
+    (void)hipFree(ctx->d_tmp);
+    (void)hipFree(ctx->d_cent);
     for (auto& ev : ctx->ev)
         if (ev) (void)hipEventDestroy(ev);
     if (ctx->own_stream) (void)hipStreamDestroy(ctx->own_stream);
@@ -371,40 +375,124 @@ int pimdl_amm_profile(pimdl_amm* a, const float* in_dev, uint32_t n, float* out_
     return PIMDL_OK;
 }
 
-int pimdl_index_calculation(pimdl_amm* a, const float* in, uint32_t n, uint16_t* idx_out, uint32_t n_stile_size,
-                            uint32_t cb_mtile_size)
+// shared tail of the two index_calculation entry points
+static int index_calc_common(Ctx* ctx, const AmmGeom& g, const float* in, const float* d_cent, uint32_t n,
+                             uint16_t* idx_out, uint32_t n_stile_size, uint32_t cb_mtile_size)
 {
-    int rc = check_run_args(a, in, idx_out, n);
-    if (rc || n == 0) return rc;
-    Ctx* ctx = a->ctx;
-    const AmmGeom& g = a->g;
-    if (!n_stile_size || !cb_mtile_size || n % n_stile_size || g.CB % cb_mtile_size)
+    if (!n_stile_size) n_stile_size = n;
+    if (!cb_mtile_size) cb_mtile_size = g.CB;
+    if (n % n_stile_size || g.CB % cb_mtile_size)
         return set_error(ctx, PIMDL_ERR_INVALID, "n_stile_size must divide n and cb_mtile_size must divide num_codebook");
+    int rc;
     const float* d_in;
     if ((rc = stage_input(ctx, g, in, n, &d_in))) return rc;
     if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, (size_t)n * g.idx_row_bytes, "hipMalloc(index scratch)"))) return rc;
     if ((rc = ensure(ctx, &ctx->d_idx16, &ctx->idx16_bytes, (size_t)n * g.CB * 2, "hipMalloc(idx16 scratch)"))) return rc;
-    if ((rc = launch_ccs(ctx, g, d_in, a->d_centroids, ctx->d_idx, n))) return rc;
+    if ((rc = launch_ccs(ctx, g, d_in, d_cent, ctx->d_idx, n))) return rc;
     if ((rc = launch_unpack_idx(ctx, g, ctx->d_idx, ctx->d_idx16, n, n_stile_size, cb_mtile_size))) return rc;
     if ((rc = hip_check(ctx, hipMemcpyAsync(idx_out, ctx->d_idx16, (size_t)n * g.CB * 2, hipMemcpyDeviceToHost, ctx->stream), "D2H idx"))) return rc;
     return hip_check(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
 }
 
-int pimdl_lut_gather(pimdl_amm* a, const uint16_t* idx, uint32_t n, float* out)
+int pimdl_amm_index_calculation(pimdl_amm* a, const float* in, uint32_t n, uint16_t* idx_out, uint32_t n_stile_size,
+                                uint32_t cb_mtile_size)
+{
+    int rc = check_run_args(a, in, idx_out, n);
+    if (rc || n == 0) return rc;
+    return index_calc_common(a->ctx, a->g, in, a->d_centroids, n, idx_out, n_stile_size, cb_mtile_size);
+}
+
+int pimdl_index_calculation(pimdl_ctx* ctx, const float* in, const float* centroids, uint32_t n, uint32_t K,
+                            uint32_t v, uint32_t C, uint16_t* idx_out, uint32_t n_stile_size, uint32_t cb_mtile_size)
+{
+    if (!ctx) return PIMDL_ERR_INVALID;
+    if (!in || !centroids || !idx_out) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_index_calculation: null buffer");
+    int rc = activate(ctx);
+    if (rc || n == 0) return rc;
+    pimdl_amm_desc d;
+    memset(&d, 0, sizeof(d));
+    d.max_n = n; d.input_feature_len = K; d.sub_vec_len = v; d.num_centroid = C; d.output_feature_len = 1;
+    d.lut_dtype = PIMDL_LUT_I8;
+    AmmGeom g;
+    memset(&g, 0, sizeof(g));
+    std::string why;
+    if (!plan_geometry(d, &g, &why)) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_index_calculation: %s", why.c_str());
+    const size_t cent_bytes = (size_t)g.CB * C * v * sizeof(float);
+    if ((rc = ensure(ctx, &ctx->d_cent, &ctx->cent_bytes, cent_bytes, "hipMalloc(centroid scratch)"))) return rc;
+    if ((rc = hip_check(ctx, hipMemcpyAsync(ctx->d_cent, centroids, cent_bytes, hipMemcpyHostToDevice, ctx->stream), "H2D centroids"))) return rc;
+    return index_calc_common(ctx, g, in, ctx->d_cent, n, idx_out, n_stile_size, cb_mtile_size);
+}
+
+static int resolve_tiling(Ctx* ctx, const AmmGeom& g, uint32_t n, const pimdl_tiling* t, pimdl_tiling* r, bool* out_identity)
+{
+    r->n_stile_size = (t && t->n_stile_size) ? t->n_stile_size : n;
+    r->cb_mtile_size = (t && t->cb_mtile_size) ? t->cb_mtile_size : g.CB;
+    r->feature_stile_size = (t && t->feature_stile_size) ? t->feature_stile_size : g.M;
+    r->feature_mtile_size = (t && t->feature_mtile_size) ? t->feature_mtile_size : r->feature_stile_size;
+    if (n % r->n_stile_size || g.CB % r->cb_mtile_size || g.M % r->feature_stile_size ||
+        r->feature_stile_size % r->feature_mtile_size)
+        return set_error(ctx, PIMDL_ERR_INVALID,
+                         "tiling does not divide the shape (n=%u ns=%u, CB=%u cm=%u, M=%u fs=%u fm=%u)", n,
+                         r->n_stile_size, g.CB, r->cb_mtile_size, g.M, r->feature_stile_size, r->feature_mtile_size);
+    *out_identity = r->n_stile_size == n && r->feature_stile_size == g.M && r->feature_mtile_size == g.M;
+    return PIMDL_OK;
+}
+
+// gather into `out` (host or device) in the requested output order
+static int gather_to(Amm* a, uint32_t n, float* out, const pimdl_tiling& til, bool out_identity)
+{
+    Ctx* ctx = a->ctx;
+    const AmmGeom& g = a->g;
+    int rc;
+    float* d_out;
+    bool out_host;
+    if ((rc = stage_output(ctx, g, out, n, &d_out, &out_host))) return rc;
+    if (out_identity) {
+        if ((rc = launch_gather(ctx, *a, ctx->d_idx, d_out, nullptr, n))) return rc;
+    } else {
+        if ((rc = ensure(ctx, &ctx->d_tmp, &ctx->tmp_bytes, (size_t)n * g.M * 4, "hipMalloc(row-major scratch)"))) return rc;
+        if ((rc = launch_gather(ctx, *a, ctx->d_idx, ctx->d_tmp, nullptr, n))) return rc;
+        if ((rc = launch_retile_output(ctx, ctx->d_tmp, d_out, n, g.M, til.n_stile_size, til.feature_stile_size,
+                                       til.feature_mtile_size)))
+            return rc;
+    }
+    return finish_output(ctx, g, out, n, out_host);
+}
+
+int pimdl_amm_run_tiled(pimdl_amm* a, const float* in, uint32_t n, float* out, const pimdl_tiling* tiling)
+{
+    int rc = check_run_args(a, in, out, n);
+    if (rc || n == 0) return rc;
+    Ctx* ctx = a->ctx;
+    pimdl_tiling til;
+    bool ident;
+    if ((rc = resolve_tiling(ctx, a->g, n, tiling, &til, &ident))) return rc;
+    const float* d_in;
+    if ((rc = stage_input(ctx, a->g, in, n, &d_in))) return rc;
+    if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, (size_t)n * a->g.idx_row_bytes, "hipMalloc(index scratch)"))) return rc;
+    if ((rc = launch_ccs(ctx, a->g, d_in, a->d_centroids, ctx->d_idx, n))) return rc;
+    return gather_to(a, n, out, til, ident);
+}
+
+int pimdl_lut_gather_tiled(pimdl_amm* a, const uint16_t* idx, uint32_t n, float* out, const pimdl_tiling* tiling)
 {
     int rc = check_run_args(a, idx, out, n);
     if (rc || n == 0) return rc;
     Ctx* ctx = a->ctx;
     const AmmGeom& g = a->g;
-    float* d_out;
-    bool out_host;
-    if ((rc = stage_output(ctx, g, out, n, &d_out, &out_host))) return rc;
+    pimdl_tiling til;
+    bool ident;
+    if ((rc = resolve_tiling(ctx, g, n, tiling, &til, &ident))) return rc;
     if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, (size_t)n * g.idx_row_bytes, "hipMalloc(index scratch)"))) return rc;
     if ((rc = ensure(ctx, &ctx->d_idx16, &ctx->idx16_bytes, (size_t)n * g.CB * 2, "hipMalloc(idx16 scratch)"))) return rc;
     if ((rc = hip_check(ctx, hipMemcpyAsync(ctx->d_idx16, idx, (size_t)n * g.CB * 2, hipMemcpyHostToDevice, ctx->stream), "H2D idx"))) return rc;
-    if ((rc = launch_pack_idx(ctx, g, ctx->d_idx16, ctx->d_idx, n))) return rc;
-    if ((rc = launch_gather(ctx, *a, ctx->d_idx, d_out, nullptr, n))) return rc;
-    return finish_output(ctx, g, out, n, out_host);
+    if ((rc = launch_pack_idx(ctx, g, ctx->d_idx16, ctx->d_idx, n, til.n_stile_size, til.cb_mtile_size))) return rc;
+    return gather_to(a, n, out, til, ident);
+}
+
+int pimdl_lut_gather(pimdl_amm* a, const uint16_t* idx, uint32_t n, float* out)
+{
+    return pimdl_lut_gather_tiled(a, idx, n, out, nullptr);
 }
 
 int pimdl_lutgen(pimdl_ctx* ctx, const float* centroids, const float* weight, uint32_t CB, uint32_t C, uint32_t v,

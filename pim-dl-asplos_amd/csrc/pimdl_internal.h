@@ -65,6 +65,10 @@ struct Ctx {
     size_t acc_bytes;
     uint16_t* d_idx16;
     size_t idx16_bytes;
+    float* d_tmp;        // row-major output before re-tiling
+    size_t tmp_bytes;
+    float* d_cent;       // centroids of a context-level pimdl_index_calculation call
+    size_t cent_bytes;
     hipEvent_t ev[4];
 };
 
@@ -78,7 +82,10 @@ int launch_gather(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, in
                   uint32_t n);
 int launch_unpack_idx(Ctx* ctx, const AmmGeom& g, const uint8_t* d_idx, uint16_t* d_idx16, uint32_t n,
                       uint32_t n_stile, uint32_t cb_mtile);
-int launch_pack_idx(Ctx* ctx, const AmmGeom& g, const uint16_t* d_idx16, uint8_t* d_idx, uint32_t n);
+int launch_pack_idx(Ctx* ctx, const AmmGeom& g, const uint16_t* d_idx16, uint8_t* d_idx, uint32_t n,
+                    uint32_t n_stile, uint32_t cb_mtile);
+int launch_retile_output(Ctx* ctx, const float* d_rowmajor, float* d_tiled, uint32_t n, uint32_t M,
+                         uint32_t n_stile, uint32_t f_stile, uint32_t f_mtile);
 int launch_lutgen_f32(Ctx* ctx, const float* d_cent, const float* d_w, float* d_lut, uint32_t CB,
                       uint32_t C, uint32_t v, uint32_t M);
 int launch_lut_quant(Ctx* ctx, const float* d_lut, int8_t* d_q, float* d_scales, uint32_t CB, uint32_t C,

@@ -1,0 +1,247 @@
+// Single-AMM driver: the counterpart of the reference's inference-engine/test/test_amm.cpp
+// (what `python run_amm.py --amm_config_file X.yaml` ends up running).
+//
+//   test_amm <kernel_config.yaml> [dpu_binary_path (ignored)] [--dump FILE] [--rounds WARMUP RECORD]
+//
+// Reads the reference's YAML keys (src/host/parser.cpp:22-47): amm_shape_params.{num_codebook,
+// num_centroid, n, input_feature_len, output_feature_len, scale, bias}, system_params.{num_threads,
+// dpu_num, nr_tasklets} and kernel_params.{n_stile_size, feature_stile_size, n_mtile_size,
+// feature_mtile_size, cb_mtile_size, feature_load_tile_size, cb_load_tile_size, lut_load_type,
+// loop_order}.  A missing kernel_params section means the identity tiling (row-major buffers).
+// Data generation follows test_amm.cpp:26-67 (mt19937(233); inputs U(-5,5), centroids and bias
+// U(-10,10), LUT uniform int8) but single-threaded, so it is reproducible.  10 warm-up and 20 timed
+// rounds of amm_host, "PIM AMM time" per round and the average, as the reference prints them
+// (test_amm.cpp:21-22,290-314).  --dump writes inputs and the output so a test can check them.
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <chrono>
+#include <fstream>
+#include <iostream>
+#include <map>
+#include <random>
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include "pimdl/amm_host.h"
+
+using namespace std;
+
+// "section.key" -> scalar text, for the two-level block YAML the reference's configs use
+static map<string, string> load_yaml(const string& path)
+{
+    map<string, string> kv;
+    ifstream f(path);
+    if (!f) {
+        cerr << "Config File Not Open" << endl;  // parser.cpp:16
+        return kv;
+    }
+    string line, section;
+    while (getline(f, line)) {
+        size_t hash = line.find('#');
+        if (hash != string::npos) line.erase(hash);
+        size_t first = line.find_first_not_of(" \t\r");
+        if (first == string::npos) continue;
+        size_t colon = line.find(':');
+        if (colon == string::npos) continue;
+        string key = line.substr(first, colon - first);
+        string val = line.substr(colon + 1);
+        size_t vb = val.find_first_not_of(" \t\r"), ve = val.find_last_not_of(" \t\r");
+        val = vb == string::npos ? "" : val.substr(vb, ve - vb + 1);
+        if (first == 0) {
+            section = key;
+            if (!val.empty()) kv[key] = val;
+        } else {
+            kv[section + "." + key] = val;
+        }
+    }
+    return kv;
+}
+
+static bool has(const map<string, string>& kv, const string& k) { return kv.count(k) != 0; }
+static uint32_t get_u32(const map<string, string>& kv, const string& k, uint32_t dflt)
+{
+    return has(kv, k) ? (uint32_t)strtoul(kv.at(k).c_str(), nullptr, 10) : dflt;
+}
+static float get_f32(const map<string, string>& kv, const string& k, float dflt)
+{
+    return has(kv, k) ? strtof(kv.at(k).c_str(), nullptr) : dflt;
+}
+
+static bool parse_amm_configs(AMMParams& p, const string& path, uint32_t* nr_tasklets)
+{
+    map<string, string> kv = load_yaml(path);
+    const char* req[] = {"amm_shape_params.n", "amm_shape_params.input_feature_len", "amm_shape_params.num_codebook",
+                         "amm_shape_params.num_centroid", "amm_shape_params.output_feature_len"};
+    for (const char* r : req)
+        if (!has(kv, r)) {
+            cerr << "Error in parsing configs: missing " << r << endl;
+            return false;
+        }
+    IndexCalcParams& ip = p.index_params;
+    LUTParams& lp = p.lut_params;
+    ip.n = get_u32(kv, "amm_shape_params.n", 0);
+    ip.input_feature_len = get_u32(kv, "amm_shape_params.input_feature_len", 0);
+    ip.num_codebook = get_u32(kv, "amm_shape_params.num_codebook", 0);
+    ip.num_centroid = get_u32(kv, "amm_shape_params.num_centroid", 0);
+    if (!ip.num_codebook || ip.input_feature_len % ip.num_codebook) {
+        cerr << "input_feature_len must be a multiple of num_codebook" << endl;  // parser.cpp:57
+        return false;
+    }
+    ip.sub_vec_len = ip.input_feature_len / ip.num_codebook;
+    ip.num_threads = get_u32(kv, "system_params.num_threads", 1);
+    ip.n_stile_size = get_u32(kv, "kernel_params.n_stile_size", ip.n);
+    ip.cb_mtile_size = get_u32(kv, "kernel_params.cb_mtile_size", ip.num_codebook);
+
+    lp.n = ip.n;
+    lp.output_feature_len = get_u32(kv, "amm_shape_params.output_feature_len", 0);
+    lp.num_codebook = ip.num_codebook;
+    lp.num_centroid = ip.num_centroid;
+    lp.scale = get_f32(kv, "amm_shape_params.scale", 1.0f);
+    lp.bias = get_f32(kv, "amm_shape_params.bias", 0.0f);
+    lp.num_threads = ip.num_threads;
+    lp.dpu_num = get_u32(kv, "system_params.dpu_num", 1);
+    lp.n_stile_size = ip.n_stile_size;
+    lp.feature_stile_size = get_u32(kv, "kernel_params.feature_stile_size", lp.output_feature_len);
+    lp.input_parallelism = lp.n / lp.n_stile_size;
+    lp.lut_parallelism = lp.output_feature_len / lp.feature_stile_size;
+    lp.n_mtile_size = get_u32(kv, "kernel_params.n_mtile_size", lp.n_stile_size);
+    lp.feature_mtile_size = get_u32(kv, "kernel_params.feature_mtile_size", lp.feature_stile_size);
+    lp.cb_mtile_size = ip.cb_mtile_size;
+    lp.feature_load_tile_size = get_u32(kv, "kernel_params.feature_load_tile_size", lp.feature_mtile_size);
+    lp.cb_load_tile_size = get_u32(kv, "kernel_params.cb_load_tile_size", lp.cb_mtile_size);
+    lp.lut_load_type = LUTLoadType(get_u32(kv, "kernel_params.lut_load_type", 0));
+    *nr_tasklets = get_u32(kv, "system_params.nr_tasklets", 16);
+
+    // the shape checks of parser.cpp:56-66 that still mean something without DPUs
+    bool ok = lp.n == lp.n_stile_size * lp.input_parallelism &&
+              lp.output_feature_len == lp.feature_stile_size * lp.lut_parallelism &&
+              lp.feature_stile_size % lp.feature_mtile_size == 0 && lp.num_codebook % lp.cb_mtile_size == 0 &&
+              lp.feature_mtile_size % lp.feature_load_tile_size == 0 && lp.cb_mtile_size % lp.cb_load_tile_size == 0;
+    if (!ok) {
+        cerr << "tiling parameters do not divide the shape" << endl;
+        return false;
+    }
+    cout << "------ amm shape params ------\n";
+    cout << "num codebook " << ip.num_codebook << ", num centroid " << ip.num_centroid << endl;
+    cout << "n " << ip.n << ", input feature len " << ip.input_feature_len << ", output feature len "
+         << lp.output_feature_len << endl;
+    cout << "scale " << lp.scale << ", bias " << lp.bias << endl;
+    cout << "------ kernel params ------\n";
+    cout << "n stile size " << lp.n_stile_size << ", feature stile size " << lp.feature_stile_size << endl;
+    cout << "feature mtile size " << lp.feature_mtile_size << ", cb mtile size " << lp.cb_mtile_size << endl;
+    cout << "lut load type " << (int)lp.lut_load_type << ", feature load tile size " << lp.feature_load_tile_size << endl;
+    cout << "sub vec len " << ip.sub_vec_len << endl;
+    return true;
+}
+
+// canonical [cb][c][M] -> the order amm_host expects (the job of reorder_pim_lut, test_amm.cpp:71-121)
+static void to_dpu_lut_order(const vector<lut_data_type>& canon, vector<lut_data_type>& dpu, const LUTParams& lp)
+{
+    const uint32_t ft = lp.lut_load_type == STATIC ? lp.feature_stile_size : lp.feature_load_tile_size;
+    const uint32_t CB = lp.num_codebook, C = lp.num_centroid, M = lp.output_feature_len;
+    for (uint32_t cb = 0; cb < CB; ++cb)
+        for (uint32_t c = 0; c < C; ++c)
+            for (uint32_t f = 0; f < M; ++f)
+                dpu[(size_t)(f / ft) * CB * C * ft + ((size_t)cb * C + c) * ft + f % ft] = canon[((size_t)cb * C + c) * M + f];
+}
+
+static double now_s()
+{
+    return chrono::duration<double>(chrono::steady_clock::now().time_since_epoch()).count();
+}
+
+int main(int argc, char** argv)
+{
+    if (argc < 2) {
+        printf("usage: %s kernel_config_yaml_path [dpu_binary_path] [--dump FILE] [--rounds WARMUP RECORD]\n", argv[0]);
+        return -1;
+    }
+    string dump_path;
+    int warmup = 10, record = 20;  // test_amm.cpp:21-22
+    for (int i = 2; i < argc; ++i) {
+        if (!strcmp(argv[i], "--dump") && i + 1 < argc) dump_path = argv[++i];
+        else if (!strcmp(argv[i], "--rounds") && i + 2 < argc) {
+            warmup = atoi(argv[++i]);
+            record = atoi(argv[++i]);
+        }
+    }
+    AMMParams amm;
+    uint32_t nr_tasklets;
+    if (!parse_amm_configs(amm, argv[1], &nr_tasklets)) return -1;
+    const IndexCalcParams& ip = amm.index_params;
+    const LUTParams& lp = amm.lut_params;
+
+    vector<float> input((size_t)ip.n * ip.input_feature_len);
+    vector<float> centroids((size_t)ip.num_codebook * ip.num_centroid * ip.sub_vec_len);
+    vector<float> bias(lp.output_feature_len);
+    vector<lut_data_type> cpu_lut((size_t)lp.num_codebook * lp.num_centroid * lp.output_feature_len), dpu_lut(cpu_lut.size());
+    vector<float> output((size_t)lp.n * lp.output_feature_len, 0.0f);
+    {
+        mt19937 gen(233);
+        uniform_real_distribution<float> di(-5.0f, 5.0f);
+        for (auto& x : input) x = di(gen);
+    }
+    {
+        mt19937 gen(233);
+        uniform_real_distribution<float> dc(-10.0f, 10.0f);
+        for (auto& x : centroids) x = dc(gen);
+    }
+    {
+        mt19937 gen(233);
+        uniform_int_distribution<int> dl(-128, 127);
+        for (auto& x : cpu_lut) x = (lut_data_type)dl(gen);
+    }
+    {
+        mt19937 gen(233);
+        uniform_real_distribution<float> db(-10.0f, 10.0f);
+        for (auto& x : bias) x = db(gen);
+    }
+    to_dpu_lut_order(cpu_lut, dpu_lut, lp);
+    cout << "data generation finished" << endl;
+
+    double t1 = now_s();
+    dpu_set_t dpu_set;
+    allocate_dpu(&dpu_set, lp.dpu_num);
+    cout << "dpu allocate time is " << now_s() - t1 << endl;
+    t1 = now_s();
+    load_binary(&dpu_set, argc > 2 && argv[2][0] != '-' ? argv[2] : "");
+    cout << "binary load time is " << now_s() - t1 << endl;
+
+    double total = 0.0;
+    for (int round = 0; round < warmup + record; ++round) {
+        cout << "---------- ROUND " << round << " ----------" << endl;
+        t1 = now_s();
+        amm_host(&dpu_set, input.data(), centroids.data(), dpu_lut.data(), bias.data(), output.data(), ip, lp);
+        double dt = now_s() - t1;
+        cout << "PIM AMM time " << dt << endl;
+        if (round >= warmup) total += dt;
+    }
+    cout << "warm up rounds " << warmup << ", record rounds " << record << endl;
+    if (record > 0) cout << "PIM AVG AMM time " << total / record << endl;
+
+    if (!dump_path.empty()) {
+        FILE* fp = fopen(dump_path.c_str(), "wb");
+        if (!fp) {
+            perror("dump");
+            return -1;
+        }
+        uint32_t hdr[12] = {ip.n, ip.input_feature_len, ip.sub_vec_len, ip.num_centroid, lp.output_feature_len,
+                            lp.n_stile_size, lp.cb_mtile_size, lp.feature_stile_size, lp.feature_mtile_size,
+                            (uint32_t)lp.lut_load_type, lp.feature_load_tile_size, lp.cb_load_tile_size};
+        fwrite(hdr, 4, 12, fp);
+        fwrite(&lp.scale, 4, 1, fp);
+        fwrite(&lp.bias, 4, 1, fp);
+        fwrite(input.data(), 4, input.size(), fp);
+        fwrite(centroids.data(), 4, centroids.size(), fp);
+        fwrite(cpu_lut.data(), 1, cpu_lut.size(), fp);
+        fwrite(bias.data(), 4, bias.size(), fp);
+        fwrite(output.data(), 4, output.size(), fp);
+        fclose(fp);
+        cout << "dumped to " << dump_path << endl;
+    }
+    free_dpu_set(&dpu_set);
+    return 0;
+}
