@@ -44,6 +44,7 @@ namespace pimdl {
 namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 
 struct Epilogue {
     float scale;
@@ -97,26 +98,59 @@ __device__ __forceinline__ void mfma_last(v4i& acc, const v4i& slot, const v4i& 
         : "v"(slot), "v"(a), "n"(WAIT));
 }
 
+// One v_mad_u32_u24: the compiler otherwise splits r*PITCH + base into a multiply and an or, and
+// every VALU instruction beyond about one per MFMA takes issue cycles away from the matrix core.
+__device__ __forceinline__ uint32_t mad24(uint32_t a, uint32_t b, uint32_t c)
+{
+    uint32_t d;
+    asm("v_mad_u32_u24 %0, %1, %2, %3" : "=v"(d) : "v"(a), "s"(b), "v"(c));
+    return d;
+}
+
+// Move one 16-byte staging unit: the register holds LUT data fetched during the previous slice and
+// is written to LDS; the same register is then re-armed with the unit of the slice after next.
+// (ds_write reads its data operand at issue; the load's result lands hundreds of cycles later.)
+__device__ __forceinline__ void stage_xfer(v4u& reg, uint32_t lds_addr, const v4u* gptr)
+{
+    asm volatile(
+        "ds_write_b128 %1, %0\n\t"
+        "global_load_dwordx4 %0, %2, off"
+        : "+v"(reg)
+        : "v"(lds_addr), "v"(gptr)
+        : "memory");
+}
+
 // C_T: centroid rows per codebook in the tiled LUT (power of two >= C)
 // Q:   16-byte chunks per row (column block = 16*Q)
 // GQ:  codebooks per lane group per slice (slice = 4*GQ codebooks)
-// TG:  16-token groups per wave (tokens per workgroup = 8 waves * TG * 16)
+// TG:  16-token groups per wave (tokens per work item = 8 waves * TG * 16)
+//
+// Persistent: the grid is a fixed number of workgroups (two per CU); workgroup w processes the work
+// items w, w + gridDim.x, ... where an item is (column block, token tile).  The loop over
+// (item, codebook slice) is one flat stream k = 0, 1, ...: while slice k is consumed from one LDS
+// buffer, the registers holding slice k+1 are written to the other buffer and re-armed with global
+// loads of slice k+2, one 16-byte unit at a time *between* groups of MFMAs, so neither the texture
+// path nor the LDS write port ever sees a burst, no wave ever stalls on issue, and the only
+// synchronisation is one barrier per slice between waves that all did identical work.
 template <int C_T, int Q, int GQ, int TG, int IDX_BITS>
-__global__ __launch_bounds__(GATHER_THREADS) void gather_i8_kernel(
+__global__ __launch_bounds__(GATHER_THREADS, 4) void gather_i8_kernel(
     const uint8_t* __restrict__ idx, const int8_t* __restrict__ lut, float* __restrict__ out,
     int32_t* __restrict__ acc_out, uint32_t N, uint32_t M, uint32_t CB_pad, uint32_t idx_row_bytes,
-    Epilogue ep)
+    uint32_t n_token_tiles, uint32_t n_items, Epilogue ep)
 {
     constexpr int G = 4 * GQ;                     // codebooks per slice
     constexpr int FB = 16 * Q;                    // columns (= bytes) per row
-    constexpr int PITCH = FB + 16;                // LDS row pitch
+    constexpr int PITCH = 16 * (Q | 1);           // LDS row pitch: an odd number of 16-byte units
     constexpr int CB_BYTES = C_T * PITCH;         // LDS bytes per codebook
     constexpr int SLICE_LDS = G * CB_BYTES;
     constexpr int SLICE_UNITS = G * C_T * Q;      // 16-byte units per slice in HBM
     constexpr int UPT = (SLICE_UNITS + GATHER_THREADS - 1) / GATHER_THREADS;
     constexpr int IDX_BYTES = GQ * IDX_BITS / 8;  // index bytes one lane needs per slice and token
+    constexpr int TOK_ITEM = GATHER_WAVES * TG * 16;
     static_assert(IDX_BYTES == 1 || IDX_BYTES == 2 || IDX_BYTES == 4, "index fetch width");
     static_assert((GQ - 1) * CB_BYTES + (Q - 1) * 16 < 65536, "ds_read immediate offset range");
+    static_assert(PITCH >= FB && (PITCH / 16) % 2 == 1, "row pitch");
+    static_assert(SLICE_UNITS % GATHER_THREADS == 0, "every lane moves the same number of staging units");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
@@ -126,32 +160,44 @@ __global__ __launch_bounds__(GATHER_THREADS) void gather_i8_kernel(
     const uint32_t g = lane >> 4;  // MFMA K-block of this lane; also selects its 4 output columns
     // codebook quarter = index of the LDS pass this lane is served in (see "Bank conflicts" above)
     const uint32_t gq = g ^ (((j + 4) >> 3) & 1);
-    const uint32_t tok0 = blockIdx.x * (GATHER_WAVES * TG * 16) + wave * (TG * 16);
-    const uint32_t colblk = blockIdx.y;
     const uint32_t nslices = CB_pad / G;
-
-    const uint4* __restrict__ lut_blk =
-        reinterpret_cast<const uint4*>(lut) + (size_t)colblk * CB_pad * C_T * Q;
+    if (blockIdx.x >= n_items) return;  // whole workgroup
+    const uint32_t my_items = (n_items - blockIdx.x + gridDim.x - 1) / gridDim.x;
+    const uint32_t total = my_items * nslices;  // length of this workgroup's (item, slice) stream
 
     // constant A operand: byte (lane % 16) of the lane's 16 bytes is 1
     const int one_hot = 1 << (8 * (j & 3));
     const v4i a_sel = {(j >> 2) == 0 ? one_hot : 0, (j >> 2) == 1 ? one_hot : 0, (j >> 2) == 2 ? one_hot : 0,
                        (j >> 2) == 3 ? one_hot : 0};
 
-    // per token group: pointer to this lane's index bytes of slice 0
-    const uint8_t* idx_ptr[TG];
-#pragma unroll
-    for (int t = 0; t < TG; ++t) {
-        uint32_t tok = tok0 + t * 16 + j;
-        if (tok >= N) tok = N - 1;  // clamp: results of such lanes are never stored
-        idx_ptr[t] = idx + (size_t)tok * idx_row_bytes + (size_t)(gq * GQ) * IDX_BITS / 8;
-    }
     auto load_idx = [](const uint8_t* base, uint32_t s) -> uint32_t {
         const uint8_t* p = base + (size_t)s * G * IDX_BITS / 8;
         if constexpr (IDX_BYTES == 4) return *reinterpret_cast<const uint32_t*>(p);
         else if constexpr (IDX_BYTES == 2) return *reinterpret_cast<const uint16_t*>(p);
         else return *p;
     };
+    // this lane's index bytes of slice 0 of an item, per token group
+    auto locate_idx = [&](uint32_t item, const uint8_t* (&ptr)[TG]) {
+        const uint32_t tok0 = (item % n_token_tiles) * TOK_ITEM + wave * (TG * 16);
+#pragma unroll
+        for (int t = 0; t < TG; ++t) {
+            uint32_t tok = tok0 + t * 16 + j;
+            if (tok >= N) tok = N - 1;  // clamp: results of such lanes are never stored
+            ptr[t] = idx + (size_t)tok * idx_row_bytes + (size_t)(gq * GQ) * IDX_BITS / 8;
+        }
+    };
+    // this lane's first staging unit of slice s of an item (the others follow GATHER_THREADS units apart)
+    auto locate_lut = [&](uint32_t item, uint32_t s) -> const v4u* {
+        return reinterpret_cast<const v4u*>(lut) + ((size_t)(item / n_token_tiles) * CB_pad * C_T * Q) +
+               (size_t)s * SLICE_UNITS + threadIdx.x;
+    };
+    // LDS byte offset (within a slice buffer) of this lane's staging unit u
+    uint32_t stage_lds[UPT];
+#pragma unroll
+    for (int u = 0; u < UPT; ++u) {
+        const uint32_t unit = threadIdx.x + u * GATHER_THREADS;
+        stage_lds[u] = (unit / Q) * PITCH + (unit % Q) * 16;
+    }
 
     v4i acc[TG][Q], slot[TG][Q];
 #pragma unroll
@@ -159,56 +205,129 @@ __global__ __launch_bounds__(GATHER_THREADS) void gather_i8_kernel(
 #pragma unroll
         for (int c = 0; c < Q; ++c) acc[t][c] = (v4i){0, 0, 0, 0};
 
-    // ---- main loop: the next slice travels HBM -> registers while the current one is consumed ----
-    uint4 stage[UPT];
+    // stream positions: p0 is consumed, p1 is written to LDS, p2 is fetched from HBM/L2
+    uint32_t item0 = blockIdx.x, s0 = 0;
+    uint32_t item1 = item0, s1 = 0, item2, s2;
+    auto advance = [&](uint32_t& item, uint32_t& s) {
+        if (++s == nslices) {
+            s = 0;
+            item += gridDim.x;
+        }
+    };
+    advance(item1, s1);
+    item2 = item1;
+    s2 = s1;
+    advance(item2, s2);
+
+    // ---- prologue: slice 0 into LDS buffer 0, slice 1 into the staging registers ----------------
+    v4u stage[UPT];
     uint32_t idx_cur[TG], idx_nxt[TG];
-#define PIMDL_FETCH_SLICE(S)                                                                        \
-    {                                                                                               \
-        const uint4* src_ = lut_blk + (size_t)(S) * SLICE_UNITS;                                    \
-        _Pragma("unroll") for (int u = 0; u < UPT; ++u)                                             \
-        {                                                                                           \
-            const uint32_t unit_ = threadIdx.x + u * GATHER_THREADS;                                \
-            stage[u] = (SLICE_UNITS % GATHER_THREADS == 0 || unit_ < SLICE_UNITS) ? src_[unit_]     \
-                                                                                  : make_uint4(0, 0, 0, 0); \
-        }                                                                                           \
-    }
-#define PIMDL_COMMIT_SLICE(BUF)                                                                     \
-    {                                                                                               \
-        unsigned char* dst_ = smem + (BUF) * SLICE_LDS;                                             \
-        _Pragma("unroll") for (int u = 0; u < UPT; ++u)                                             \
-        {                                                                                           \
-            const uint32_t unit_ = threadIdx.x + u * GATHER_THREADS;                                \
-            if (SLICE_UNITS % GATHER_THREADS == 0 || unit_ < SLICE_UNITS)                           \
-                *reinterpret_cast<uint4*>(dst_ + (unit_ / Q) * PITCH + (unit_ % Q) * 16) = stage[u]; \
-        }                                                                                           \
-    }
-    PIMDL_FETCH_SLICE(0)
+    const uint8_t* idx_base[TG];  // of the item p1 belongs to
+    {
+        const v4u* src = locate_lut(item0, 0);
 #pragma unroll
-    for (int t = 0; t < TG; ++t) idx_cur[t] = load_idx(idx_ptr[t], 0);
-    PIMDL_COMMIT_SLICE(0)
+        for (int u = 0; u < UPT; ++u) stage[u] = src[u * GATHER_THREADS];
+        locate_idx(item0, idx_base);
+#pragma unroll
+        for (int t = 0; t < TG; ++t) idx_cur[t] = load_idx(idx_base[t], 0);
+#pragma unroll
+        for (int u = 0; u < UPT; ++u) *reinterpret_cast<v4u*>(smem + stage_lds[u]) = stage[u];
+        const bool valid1 = 1 < total;
+        src = valid1 ? locate_lut(item1, s1) : locate_lut(item0, 0);
+#pragma unroll
+        for (int u = 0; u < UPT; ++u) stage[u] = src[u * GATHER_THREADS];
+        if (valid1 && s1 == 0) locate_idx(item1, idx_base);
+    }
     __syncthreads();
 
     const uint32_t lane_base = gq * GQ * CB_BYTES;
-    for (uint32_t s = 0; s < nslices; ++s) {
-        // the last iteration re-fetches its own slice (into the idle buffer) instead of branching
-        const uint32_t sn = s + 1 < nslices ? s + 1 : s;
-        PIMDL_FETCH_SLICE(sn)
+    bool pending_epilogue = false;
+    uint32_t epilogue_item = 0;
+
+    // De-quantise and store one finished item, then clear the accumulators.  Lane (j, g) holds columns
+    // 4*g .. 4*g+3 of every 16-column chunk for token j.  It runs right after a top-of-slice wait, so
+    // its stores have a whole slice to drain before anything waits on the memory counter again; the
+    // bias values are fetched first so that no store sits between a load and its use.
+    auto epilogue = [&](uint32_t item) {
+        const uint32_t colblk = item / n_token_tiles;
+        const uint32_t tok0 = (item % n_token_tiles) * TOK_ITEM + wave * (TG * 16);
+        const bool vec_store = (M % 4 == 0);
+        float4 bv[Q];
 #pragma unroll
-        for (int t = 0; t < TG; ++t) idx_nxt[t] = load_idx(idx_ptr[t], sn);
-        // keep the prefetch of the next slice (and of its indices) at the top of the iteration
-        __builtin_amdgcn_sched_barrier(0);
-        const uint32_t buf = (s & 1) * SLICE_LDS + lane_base;
-        // LDS byte address of the row each token group gathers from, for every codebook of the quarter
+        for (int c = 0; c < Q; ++c) {
+            const uint32_t f = colblk * FB + c * 16 + 4 * g;
+            bv[c] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (ep.bias && f < M) {
+                if (vec_store) {
+                    bv[c] = *reinterpret_cast<const float4*>(ep.bias + f);
+                } else {
+                    bv[c].x = ep.bias[f];
+                    if (f + 1 < M) bv[c].y = ep.bias[f + 1];
+                    if (f + 2 < M) bv[c].z = ep.bias[f + 2];
+                    if (f + 3 < M) bv[c].w = ep.bias[f + 3];
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < TG; ++t) {
+            const uint32_t tok = tok0 + t * 16 + j;
+#pragma unroll
+            for (int c = 0; c < Q; ++c) {
+                const uint32_t f = colblk * FB + c * 16 + 4 * g;
+                const v4i a = acc[t][c];
+                acc[t][c] = (v4i){0, 0, 0, 0};
+                if (tok >= N || f >= M) continue;
+                float4 o;
+                o.x = dequant(a[0], ep.scale, ep.lut_bias_term, bv[c].x);
+                o.y = dequant(a[1], ep.scale, ep.lut_bias_term, bv[c].y);
+                o.z = dequant(a[2], ep.scale, ep.lut_bias_term, bv[c].z);
+                o.w = dequant(a[3], ep.scale, ep.lut_bias_term, bv[c].w);
+                if (vec_store) {  // M % 4 == 0 and f % 4 == 0: the whole float4 is in range and aligned
+                    *reinterpret_cast<float4*>(out + (size_t)tok * M + f) = o;
+                    if (acc_out) *reinterpret_cast<v4i*>(acc_out + (size_t)tok * M + f) = a;
+                } else {
+                    const float ov[4] = {o.x, o.y, o.z, o.w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (f + e < M) {
+                            out[(size_t)tok * M + f + e] = ov[e];
+                            if (acc_out) acc_out[(size_t)tok * M + f + e] = a[e];
+                        }
+                    }
+                }
+            }
+        }
+    };
+
+    for (uint32_t k = 0; k < total; ++k) {
+        // everything this lane has in flight is at least one slice old: the staging registers hold
+        // slice k+1, the indices fetched during the previous iteration have landed
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (pending_epilogue) {  // workgroup-uniform
+            epilogue(epilogue_item);
+            pending_epilogue = false;
+        }
+
+        const bool valid1 = k + 1 < total, valid2 = k + 2 < total;  // workgroup-uniform
+#pragma unroll
+        for (int t = 0; t < TG; ++t) idx_nxt[t] = load_idx(idx_base[t], valid1 ? s1 : 0);
+        const v4u* fetch_ptr = valid2 ? locate_lut(item2, s2) : locate_lut(item0, s0);
+
+        const uint32_t buf = (k & 1) * SLICE_LDS + lane_base;
+        const uint32_t wbuf = ((k + 1) & 1) * SLICE_LDS;
+        // LDS byte address of the row each token group gathers from, per codebook of the quarter
         uint32_t row_addr[GQ][TG];
 #pragma unroll
         for (int q = 0; q < GQ; ++q)
 #pragma unroll
             for (int t = 0; t < TG; ++t)
-                row_addr[q][t] = buf + ((idx_cur[t] >> (IDX_BITS * q)) & ((1u << IDX_BITS) - 1)) * PITCH;
+                row_addr[q][t] = mad24((idx_cur[t] >> (IDX_BITS * q)) & ((1u << IDX_BITS) - 1), PITCH, buf);
+
         // Rolling pipeline, one register slot per accumulator: the row piece for (q+1, t, c) is
         // requested into the slot as soon as the MFMA for (q, t, c) has consumed it, so TG*Q reads
-        // stay in flight behind the matrix core.  Waits are explicit: LDS returns in order, and
-        // lgkmcnt(TG*Q-1) before an MFMA means "the oldest outstanding read has landed".
+        // stay in flight behind the matrix core.  Waits are explicit: LDS operations complete in
+        // order, and lgkmcnt(TG*Q-1) before an MFMA means "the oldest outstanding read has landed"
+        // (an interleaved staging write only makes that wait stricter).
         static_for<0, TG * Q>([&](auto i) {
             constexpr int t = i / Q, c = i % Q;
             lds_read<c * 16>(slot[t][c], row_addr[0][t]);
@@ -219,52 +338,42 @@ __global__ __launch_bounds__(GATHER_THREADS) void gather_i8_kernel(
                 mfma_then_read<(q + 1) * CB_BYTES + c * 16, TG * Q - 1>(acc[t][c], slot[t][c], a_sel,
                                                                        row_addr[q + 1][t]);
             });
+            // staging units of this step: UPT units spread over the GQ-1 interior steps
+            static_for<(q * UPT) / (GQ - 1), ((q + 1) * UPT) / (GQ - 1)>([&](auto u) {
+                stage_xfer(stage[u], wbuf + stage_lds[u], fetch_ptr + u * GATHER_THREADS);
+            });
         });
+        if constexpr (GQ == 1) {
+            static_for<0, UPT>([&](auto u) {
+                stage_xfer(stage[u], wbuf + stage_lds[u], fetch_ptr + u * GATHER_THREADS);
+            });
+        }
         static_for<0, TG * Q>([&](auto i) {
             constexpr int t = i / Q, c = i % Q;
             mfma_last<TG * Q - 1 - i>(acc[t][c], slot[t][c], a_sel);
         });
-        PIMDL_COMMIT_SLICE((s + 1) & 1)
+
 #pragma unroll
         for (int t = 0; t < TG; ++t) idx_cur[t] = idx_nxt[t];
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this lane's staging writes are in LDS
         __syncthreads();
-    }
-#undef PIMDL_FETCH_SLICE
-#undef PIMDL_COMMIT_SLICE
 
-    // ---- epilogue: lane (j, g) holds columns 4*g .. 4*g+3 of every 16-column chunk for token j ----
-    const bool vec_store = (M % 4 == 0);
-#pragma unroll
-    for (int t = 0; t < TG; ++t) {
-        const uint32_t tok = tok0 + t * 16 + j;
-        if (tok >= N) continue;
-#pragma unroll
-        for (int c = 0; c < Q; ++c) {
-            const uint32_t f = colblk * FB + c * 16 + 4 * g;
-            if (f >= M) continue;
-            const v4i a = acc[t][c];
-            if (vec_store) {  // M % 4 == 0 and f % 4 == 0: the whole float4 is in range and aligned
-                float4 bv = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (ep.bias) bv = *reinterpret_cast<const float4*>(ep.bias + f);
-                float4 o;
-                o.x = dequant(a[0], ep.scale, ep.lut_bias_term, bv.x);
-                o.y = dequant(a[1], ep.scale, ep.lut_bias_term, bv.y);
-                o.z = dequant(a[2], ep.scale, ep.lut_bias_term, bv.z);
-                o.w = dequant(a[3], ep.scale, ep.lut_bias_term, bv.w);
-                *reinterpret_cast<float4*>(out + (size_t)tok * M + f) = o;
-                if (acc_out) *reinterpret_cast<v4i*>(acc_out + (size_t)tok * M + f) = a;
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    if (f + e < M) {
-                        const float b = ep.bias ? ep.bias[f + e] : 0.0f;
-                        out[(size_t)tok * M + f + e] = dequant(a[e], ep.scale, ep.lut_bias_term, b);
-                        if (acc_out) acc_out[(size_t)tok * M + f + e] = a[e];
-                    }
-                }
-            }
+        if (s0 + 1 == nslices) {  // item finished: its epilogue runs after the next top-of-slice wait
+            pending_epilogue = true;
+            epilogue_item = item0;
         }
+
+        // advance the three stream positions
+        item0 = item1;
+        s0 = s1;
+        item1 = item2;
+        s1 = s2;
+        advance(item2, s2);
+        if (k + 2 < total && s1 == 0) locate_idx(item1, idx_base);  // p1 entered a new item
     }
+    // drain the loads armed by the last iterations before the registers die, then the last item
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (pending_epilogue) epilogue(epilogue_item);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -379,8 +488,9 @@ template <int C_T, int Q, int GQ, int TG, int IDX_BITS>
 int launch_i8(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_t* d_acc, uint32_t n,
               const Epilogue& ep)
 {
-    constexpr int TOK_WG = GATHER_WAVES * TG * 16;
-    constexpr int LDS = 2 * 4 * GQ * C_T * (16 * Q + 16);
+    constexpr int TOK_ITEM = GATHER_WAVES * TG * 16;
+    constexpr int PITCH = 16 * (Q | 1);
+    constexpr int LDS = 2 * 4 * GQ * C_T * PITCH;
     auto kern = gather_i8_kernel<C_T, Q, GQ, TG, IDX_BITS>;
     static bool attr_set = false;
     if (!attr_set) {
@@ -390,10 +500,15 @@ int launch_i8(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_
         if (rc) return rc;
         attr_set = true;
     }
-    dim3 grid((n + TOK_WG - 1) / TOK_WG, a.g.M_pad / (16 * Q));
-    hipLaunchKernelGGL(kern, grid, dim3(GATHER_THREADS), LDS, ctx->stream, d_idx,
+    const uint32_t n_token_tiles = (n + TOK_ITEM - 1) / TOK_ITEM;
+    const uint32_t n_items = n_token_tiles * (a.g.M_pad / (16 * Q));
+    // persistent grid: as many workgroups as fit at once (LDS-limited), never more than there are items
+    const uint32_t per_cu = LDS > 0 ? (uint32_t)(ctx->prop.maxSharedMemoryPerMultiProcessor / LDS) : 1;
+    uint32_t grid = ctx->prop.multiProcessorCount * (per_cu < 1 ? 1 : per_cu > 2 ? 2 : per_cu);
+    if (grid > n_items) grid = n_items;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(GATHER_THREADS), LDS, ctx->stream, d_idx,
                        reinterpret_cast<const int8_t*>(a.d_lut), d_out, d_acc, n, a.g.M, a.g.CB_pad,
-                       a.g.idx_row_bytes, ep);
+                       a.g.idx_row_bytes, n_token_tiles, n_items, ep);
     return hip_check(ctx, hipGetLastError(), "gather_i8_kernel launch");
 }
 
