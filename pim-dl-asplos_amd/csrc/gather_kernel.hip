@@ -120,6 +120,15 @@ __device__ __forceinline__ void stage_xfer(v4u& reg, uint32_t lds_addr, const v4
         : "memory");
 }
 
+// index fetch of 1, 2 or 4 bytes (zero-extended) that the compiler does not know is in flight
+template <int BYTES>
+__device__ __forceinline__ void load_idx_async(uint32_t& reg, const void* gptr)
+{
+    if constexpr (BYTES == 4) asm volatile("global_load_dword %0, %1, off" : "=v"(reg) : "v"(gptr) : "memory");
+    else if constexpr (BYTES == 2) asm volatile("global_load_ushort %0, %1, off" : "=v"(reg) : "v"(gptr) : "memory");
+    else asm volatile("global_load_ubyte %0, %1, off" : "=v"(reg) : "v"(gptr) : "memory");
+}
+
 // C_T: centroid rows per codebook in the tiled LUT (power of two >= C)
 // Q:   16-byte chunks per row (column block = 16*Q)
 // GQ:  codebooks per lane group per slice (slice = 4*GQ codebooks)
@@ -229,7 +238,7 @@ __global__ __launch_bounds__(GATHER_THREADS, 4) void gather_i8_kernel(
         for (int u = 0; u < UPT; ++u) stage[u] = src[u * GATHER_THREADS];
         locate_idx(item0, idx_base);
 #pragma unroll
-        for (int t = 0; t < TG; ++t) idx_cur[t] = load_idx(idx_base[t], 0);
+        for (int t = 0; t < TG; ++t) idx_nxt[t] = load_idx(idx_base[t], 0);  // moved to idx_cur at the top of k = 0
 #pragma unroll
         for (int u = 0; u < UPT; ++u) *reinterpret_cast<v4u*>(smem + stage_lds[u]) = stage[u];
         const bool valid1 = 1 < total;
@@ -302,7 +311,16 @@ __global__ __launch_bounds__(GATHER_THREADS, 4) void gather_i8_kernel(
     for (uint32_t k = 0; k < total; ++k) {
         // everything this lane has in flight is at least one slice old: the staging registers hold
         // slice k+1, the indices fetched during the previous iteration have landed
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        // (the indices move out of their in-flight registers inside the asm, behind the wait, so the
+        // compiler never holds a value it could copy before it has landed)
+        static_assert(TG == 1 || TG == 2, "operand list of the wait below");
+        if constexpr (TG == 2)
+            asm volatile("s_waitcnt vmcnt(0)\n\tv_mov_b32 %0, %2\n\tv_mov_b32 %1, %3"
+                         : "=&v"(idx_cur[0]), "=&v"(idx_cur[1])
+                         : "v"(idx_nxt[0]), "v"(idx_nxt[1])
+                         : "memory");
+        else
+            asm volatile("s_waitcnt vmcnt(0)\n\tv_mov_b32 %0, %1" : "=&v"(idx_cur[0]) : "v"(idx_nxt[0]) : "memory");
         if (pending_epilogue) {  // workgroup-uniform
             epilogue(epilogue_item);
             pending_epilogue = false;
@@ -310,7 +328,8 @@ __global__ __launch_bounds__(GATHER_THREADS, 4) void gather_i8_kernel(
 
         const bool valid1 = k + 1 < total, valid2 = k + 2 < total;  // workgroup-uniform
 #pragma unroll
-        for (int t = 0; t < TG; ++t) idx_nxt[t] = load_idx(idx_base[t], valid1 ? s1 : 0);
+        for (int t = 0; t < TG; ++t)
+            load_idx_async<IDX_BYTES>(idx_nxt[t], idx_base[t] + (size_t)(valid1 ? s1 : 0) * G * IDX_BITS / 8);
         const v4u* fetch_ptr = valid2 ? locate_lut(item2, s2) : locate_lut(item0, s0);
 
         const uint32_t buf = (k & 1) * SLICE_LDS + lane_base;
@@ -338,8 +357,9 @@ __global__ __launch_bounds__(GATHER_THREADS, 4) void gather_i8_kernel(
                 mfma_then_read<(q + 1) * CB_BYTES + c * 16, TG * Q - 1>(acc[t][c], slot[t][c], a_sel,
                                                                        row_addr[q + 1][t]);
             });
-            // staging units of this step: UPT units spread over the GQ-1 interior steps
-            static_for<(q * UPT) / (GQ - 1), ((q + 1) * UPT) / (GQ - 1)>([&](auto u) {
+            // staging: one unit after each of the first steps (the rest after the last interior step),
+            // so that the re-armed loads have most of a slice to land
+            static_for<(q < UPT ? q : UPT), (q + 1 == GQ - 1 ? UPT : (q + 1 < UPT ? q + 1 : UPT))>([&](auto u) {
                 stage_xfer(stage[u], wbuf + stage_lds[u], fetch_ptr + u * GATHER_THREADS);
             });
         });
@@ -353,8 +373,6 @@ __global__ __launch_bounds__(GATHER_THREADS, 4) void gather_i8_kernel(
             mfma_last<TG * Q - 1 - i>(acc[t][c], slot[t][c], a_sel);
         });
 
-#pragma unroll
-        for (int t = 0; t < TG; ++t) idx_cur[t] = idx_nxt[t];
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this lane's staging writes are in LDS
         __syncthreads();
 
@@ -543,7 +561,7 @@ int launch_f32(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, uint3
 //   64    (4, 2)  40 KB                      (4, 8)  40 KB
 //   128   (2, 2)  48 KB                      (2, 8)  48 KB
 //   256   (2, 1)  48 KB                      (2, 4)  48 KB
-bool plan_geometry(const pimdl_amm_desc& d, AmmGeom* g, std::string* why)
+bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::string* why)
 {
     const uint32_t K = d.input_feature_len, v = d.sub_vec_len, C = d.num_centroid, M = d.output_feature_len;
     if (!K || !v || !C || !M || !d.max_n) { *why = "zero-sized dimension"; return false; }
@@ -560,6 +578,24 @@ bool plan_geometry(const pimdl_amm_desc& d, AmmGeom* g, std::string* why)
     g->idx_row_bytes = g->CB_pad * g->idx_bits / 8;
     const bool i8 = d.lut_dtype == PIMDL_LUT_I8;
     g->q = ct >= 128 ? 2 : 4;
+    if (i8 && ct >= 16 && ct <= 64) {
+        // Column block of 64 or 48 columns: take the one that fills the persistent grid (two
+        // workgroups per CU) more evenly for the largest batch this operator will see.  An item is
+        // 256 tokens x one column block; all items cost the same.
+        const uint32_t slots = 2 * (num_cus ? num_cus : 256);
+        const uint32_t tiles = (d.max_n + 255) / 256;
+        double best = -1.0;
+        for (uint32_t q : {4u, 3u}) {
+            const uint32_t blocks = (M + 16 * q - 1) / (16 * q);
+            const uint64_t items = (uint64_t)tiles * blocks;
+            const uint64_t rounds = (items + slots - 1) / slots;
+            const double eff = (double)items / (double)(rounds * slots) * (double)M / (double)(blocks * 16 * q);
+            if (eff > best + 1e-9) {
+                best = eff;
+                g->q = q;
+            }
+        }
+    }
     if (i8) {
         g->gq = ct <= 16 ? 8 : ct == 32 ? 4 : ct <= 128 ? 2 : 1;
         g->cb_per_slice = 4 * g->gq;
@@ -573,7 +609,7 @@ bool plan_geometry(const pimdl_amm_desc& d, AmmGeom* g, std::string* why)
         g->gather_threads = GF_THREADS;
         g->tokens_per_wg = GF_THREADS;
     }
-    g->row_pitch = 16 * g->q + 16;
+    g->row_pitch = 16 * (g->q | 1);
     g->gather_lds_bytes = 2 * g->cb_per_slice * ct * g->row_pitch;
     g->M_pad = (M + g->col_block - 1) / g->col_block * g->col_block;
     g->ccs_cb_per_wg = ccs_cb_per_wg(v);
@@ -593,9 +629,15 @@ int launch_gather(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, in
         ep.bias = a.d_bias;
         switch (g.C_tile) {
             case 8: return launch_i8<8, 4, 8, 2, 4>(ctx, a, d_idx, d_out, d_acc, n, ep);
-            case 16: return launch_i8<16, 4, 8, 2, 4>(ctx, a, d_idx, d_out, d_acc, n, ep);
-            case 32: return launch_i8<32, 4, 4, 2, 8>(ctx, a, d_idx, d_out, d_acc, n, ep);
-            case 64: return launch_i8<64, 4, 2, 2, 8>(ctx, a, d_idx, d_out, d_acc, n, ep);
+            case 16:
+                return g.q == 3 ? launch_i8<16, 3, 8, 2, 4>(ctx, a, d_idx, d_out, d_acc, n, ep)
+                                : launch_i8<16, 4, 8, 2, 4>(ctx, a, d_idx, d_out, d_acc, n, ep);
+            case 32:
+                return g.q == 3 ? launch_i8<32, 3, 4, 2, 8>(ctx, a, d_idx, d_out, d_acc, n, ep)
+                                : launch_i8<32, 4, 4, 2, 8>(ctx, a, d_idx, d_out, d_acc, n, ep);
+            case 64:
+                return g.q == 3 ? launch_i8<64, 3, 2, 2, 8>(ctx, a, d_idx, d_out, d_acc, n, ep)
+                                : launch_i8<64, 4, 2, 2, 8>(ctx, a, d_idx, d_out, d_acc, n, ep);
             case 128: return launch_i8<128, 2, 2, 2, 8>(ctx, a, d_idx, d_out, d_acc, n, ep);
             case 256: return launch_i8<256, 2, 1, 2, 8>(ctx, a, d_idx, d_out, d_acc, n, ep);
         }

@@ -234,7 +234,7 @@ int pimdl_amm_create(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const float* ce
     AmmGeom g;
     memset(&g, 0, sizeof(g));
     std::string why;
-    if (!plan_geometry(*desc, &g, &why)) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_create: %s", why.c_str());
+    if (!plan_geometry(*desc, ctx->prop.multiProcessorCount, &g, &why)) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_create: %s", why.c_str());
     const bool i8 = desc->lut_dtype == PIMDL_LUT_I8;
     if (i8 && !scales) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_create: int8 LUT needs scales");
     if (i8 && desc->scale_group != 0)
@@ -416,7 +416,7 @@ int pimdl_index_calculation(pimdl_ctx* ctx, const float* in, const float* centro
     AmmGeom g;
     memset(&g, 0, sizeof(g));
     std::string why;
-    if (!plan_geometry(d, &g, &why)) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_index_calculation: %s", why.c_str());
+    if (!plan_geometry(d, ctx->prop.multiProcessorCount, &g, &why)) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_index_calculation: %s", why.c_str());
     const size_t cent_bytes = (size_t)g.CB * C * v * sizeof(float);
     if ((rc = ensure(ctx, &ctx->d_cent, &ctx->cent_bytes, cent_bytes, "hipMalloc(centroid scratch)"))) return rc;
     if ((rc = hip_check(ctx, hipMemcpyAsync(ctx->d_cent, centroids, cent_bytes, hipMemcpyHostToDevice, ctx->stream), "H2D centroids"))) return rc;

@@ -93,6 +93,6 @@ int launch_lut_quant(Ctx* ctx, const float* d_lut, int8_t* d_q, float* d_scales,
 int launch_diag(Ctx* ctx, uint64_t bytes, float* copy_gbps, float* lds_gbps);
 
 uint32_t ccs_cb_per_wg(uint32_t v);  // codebooks one ccs workgroup covers (0: generic kernel)
-bool plan_geometry(const pimdl_amm_desc& d, AmmGeom* g, std::string* why);
+bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::string* why);
 
 }  // namespace pimdl
