@@ -11,13 +11,37 @@
 //   * the compare `(double)(best - d) > 1e-6` equals the fp32 compare `(best - d) > 1e-6f`,
 //     because (float)1e-6 < 1e-6 < nextafter((float)1e-6).
 //
-// Mapping.  One lane owns one token; a workgroup of 256 lanes owns 256 tokens x CBT codebooks.
-// The activation tile is loaded from HBM with fully coalesced 16-byte loads, transposed through
+// Mapping.  One lane owns one token.  A workgroup of four waves owns a tile of 64 tokens x
+// 4*CBT codebooks: wave w searches the w-th group of CBT codebooks for all 64 tokens.  A tile row
+// is 512 contiguous bytes in HBM (v <= 16), loaded with coalesced 16-byte loads, transposed through
 // LDS (row pitch padded by 16 B so the per-lane 16-byte reads hit distinct banks), and each lane
-// keeps its row slice in registers.  Centroids are wave-uniform, so the compiler fetches them with
-// scalar loads and feeds them to the VALU as SGPR operands: no VGPRs, no LDS traffic for them.
+// keeps its 32-float row slice in registers.  Workgroups are persistent and fetch the next tile
+// into registers before searching the current one.  In the exact scan centroids are wave-uniform
+// and arrive as SGPR operands through scalar loads.
 // Indices leave packed (4 bits when C <= 16, else 8) so the gather reads them once.
+//
+// Two-speed search.  The scan above costs 3v+3 VALU operations per centroid.  Almost every
+// (token, codebook) pair has a nearest centroid that wins by far more than rounding error plus the
+// 1e-6 hysteresis, and for those the scan returns the true nearest centroid whatever the order.  So
+// each lane first evaluates the expanded form  |x|^2 + |c|^2 - 2 x.c  with FMAs (v+1 operations per
+// centroid; -2c and |c|^2 are precomputed per operator and arrive as SGPR operands), keeps the two
+// smallest values with the centroid id packed into the low mantissa bits (v_and_or, v_med3,
+// v_min: 3 operations), and accepts the winner only when
+//     second - best  >  2 * (error bound of both formulas + packing error) + 1e-6 .
+// If any lane of the wave fails that test (near ties, non-finite data) the whole wave replays the
+// reference's exact scan for that codebook, so the output is bit-identical in every case.
+//
+// Error bound.  u = 2^-24.  With XX = sum x_t^2, CN = sum c_t^2 and D the real-valued distance
+// (D <= 2(XX+CN)): the reference chain has relative error <= (v+2)u, i.e. <= 2(v+2)u(XX+CN);
+// the FMA form accumulates <= (3v+1)u(XX+CN) (v roundings in each of XX and CN, one for their sum,
+// v for the FMAs whose partial sums stay below 2(XX+CN)).  Sum: (5v+5)u(XX+CN); the kernel uses
+// three times that.  Packing the id into the low IDX_BITS bits moves a value by less than
+// 2^IDX_BITS ulp, i.e. 2^(IDX_BITS-22) |value|, charged against the second-smallest value.
 #include "pimdl_internal.h"
+
+#include <stdlib.h>
+
+#include <type_traits>
 
 namespace pimdl {
 
@@ -27,62 +51,137 @@ template <int V>
 struct CcsShape {
     static constexpr int ROW_FLOATS = (2 * V > 32) ? 2 * V : 32;  // floats of one token per tile
     static constexpr int CBT = ROW_FLOATS / V;                    // codebooks per workgroup
-    static constexpr int PITCH = ROW_FLOATS + 4;                  // floats; +16 B: conflict-free b128
+    static constexpr int WAVES = 4;                               // each wave: its own codebook group
+    static constexpr int TILE_TOKENS = 64;                        // one token per lane
+    static constexpr int PITCH = WAVES * ROW_FLOATS + 4;          // floats; +16 B: conflict-free b128
+    static constexpr int LDS_BYTES = TILE_TOKENS * PITCH * 4;
 };
 
 constexpr int CCS_THREADS = 256;
 
-template <int V, int IDX_BITS>
-__global__ __launch_bounds__(CCS_THREADS) void ccs_kernel(const float* __restrict__ x,
-                                                         const float* __restrict__ cent,
-                                                         uint8_t* __restrict__ idx, uint32_t N,
-                                                         uint32_t K, uint32_t CB, uint32_t C,
-                                                         uint32_t idx_row_bytes, int vec_ok)
+inline size_t ccs_aux_floats(const AmmGeom& g)
 {
-    using S = CcsShape<V>;
-    constexpr int RF = S::ROW_FLOATS, CBT = S::CBT, PITCH = S::PITCH;
-    __shared__ __attribute__((aligned(16))) float tile[CCS_THREADS * PITCH];
+    return (size_t)g.CB * (g.v + 1) * ((g.C + 15) / 16 * 16);
+}
 
-    const uint32_t tok0 = blockIdx.x * CCS_THREADS;
-    const uint32_t cb0 = blockIdx.y * CBT;
-    const uint32_t col0 = cb0 * V;
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f)
+{
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1>{});
+    }
+}
 
-    // ---- stage the [256 tokens][RF floats] tile, coalesced along the row --------------------
-    constexpr int F4_PER_ROW = RF / 4;
-    constexpr int ROWS_PER_PASS = CCS_THREADS / F4_PER_ROW;
-    {
-        const uint32_t q = threadIdx.x % F4_PER_ROW;
-        const uint32_t r0 = threadIdx.x / F4_PER_ROW;
-#pragma unroll 4
-        for (uint32_t r = r0; r < CCS_THREADS; r += ROWS_PER_PASS) {
-            uint32_t tok = tok0 + r;
-            if (tok >= N) tok = N - 1;  // rows past N repeat the last token; never stored
-            const uint32_t col = col0 + 4 * q;
-            float4 val;
-            const float* src = x + (size_t)tok * K + col;
-            if (vec_ok && col + 4 <= K) {
-                val = *reinterpret_cast<const float4*>(src);
-            } else {
-                val.x = (col + 0 < K) ? src[0] : 0.0f;
-                val.y = (col + 1 < K) ? src[1] : 0.0f;
-                val.z = (col + 2 < K) ? src[2] : 0.0f;
-                val.w = (col + 3 < K) ? src[3] : 0.0f;
+// Derived centroid data behind the raw [CB][C][v] block of a centroid buffer (C16 = C rounded up
+// to a multiple of 16):
+//   aux   [CB][v+1][C16] = rows t < v: -2 c_t, row v: |c|^2; centroids past C hold (0, 3e38) so
+//                          they can be evaluated like real ones and never win
+//   cnmax [CB]           = max_c |c|^2, NaN when any centroid of the codebook is not finite or so
+//                          large that the fast form could overflow (forces the exact scan)
+__global__ void ccs_prep_kernel(const float* __restrict__ cent, float* __restrict__ aux,
+                                float* __restrict__ cnmax, uint32_t C, uint32_t v)
+{
+    __shared__ float cn_s[256];
+    const uint32_t cb = blockIdx.x;
+    const uint32_t C16 = (C + 15) / 16 * 16;
+    float* ap = aux + (size_t)cb * (v + 1) * C16;
+    for (uint32_t c = threadIdx.x; c < C16; c += blockDim.x) {
+        float cn = 3e38f;
+        if (c < C) {
+            const float* cp = cent + ((size_t)cb * C + c) * v;
+            cn = 0.0f;
+            for (uint32_t t = 0; t < v; ++t) {
+                cn = fmaf(cp[t], cp[t], cn);
+                ap[(size_t)t * C16 + c] = -2.0f * cp[t];
             }
-            *reinterpret_cast<float4*>(&tile[r * PITCH + 4 * q]) = val;
+            cn_s[c] = cn;
+        } else {
+            for (uint32_t t = 0; t < v; ++t) ap[(size_t)t * C16 + c] = 0.0f;
         }
+        ap[(size_t)v * C16 + c] = cn;
     }
     __syncthreads();
+    if (threadIdx.x == 0) {
+        float m = 0.0f;
+        bool bad = false;
+        for (uint32_t c = 0; c < C; ++c) {
+            const float cn = cn_s[c];
+            if (!(cn < 1e36f)) bad = true;
+            m = fmaxf(m, cn);
+        }
+        cnmax[cb] = bad ? __builtin_nanf("") : m;
+    }
+}
 
-    // ---- each lane takes its own row into registers --------------------------------------------
+template <int V, int IDX_BITS, bool FAST>
+__global__ __launch_bounds__(CCS_THREADS) void ccs_kernel(const float* __restrict__ x,
+                                                         const float* __restrict__ cent,
+                                                         const float* __restrict__ aux,
+                                                         const float* __restrict__ cnmax,
+                                                         uint8_t* __restrict__ idx, uint32_t N,
+                                                         uint32_t K, uint32_t CB, uint32_t C,
+                                                         uint32_t idx_row_bytes, int vec_ok,
+                                                         uint32_t CB_pad, uint32_t tiles_cb,
+                                                         uint32_t total_tiles)
+{
+    using S = CcsShape<V>;
+    constexpr int RF = S::ROW_FLOATS, CBT = S::CBT, PITCH = S::PITCH, TT = S::TILE_TOKENS;
+    static_assert(S::WAVES * 64 == CCS_THREADS, "one wave per codebook group");
+    __shared__ __attribute__((aligned(16))) float tile[TT * PITCH];
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+
+    // ---- persistent loop over (token tile, codebook group) tiles; the next tile's activations
+    //      are fetched into registers before the current tile is searched, so HBM latency and
+    //      bandwidth hide under the VALU work -----------------------------------------------------
+    // A tile is 64 tokens x 4*RF floats: rows of 4*RF*4 bytes (512 B for v <= 16) are contiguous in
+    // HBM, and wave w searches the w-th quarter of the columns for all 64 tokens.
+    constexpr int F4_PER_ROW = S::WAVES * RF / 4;
+    constexpr int ROWS_PER_PASS = CCS_THREADS / F4_PER_ROW;
+    constexpr int PASSES = TT / ROWS_PER_PASS;                // float4 per lane per tile (= RF / 4)
+    const uint32_t fq = threadIdx.x % F4_PER_ROW;
+    const uint32_t fr0 = threadIdx.x / F4_PER_ROW;
+    auto fetch = [&](float4 (&pf)[PASSES], uint32_t tile_id) {
+        const uint32_t t_tok0 = (tile_id / tiles_cb) * TT;
+        const uint32_t col = (tile_id % tiles_cb) * (S::WAVES * RF) + 4 * fq;
+#pragma unroll
+        for (int i = 0; i < PASSES; ++i) {
+            uint32_t tok = t_tok0 + fr0 + i * ROWS_PER_PASS;
+            if (tok >= N) tok = N - 1;  // rows past N repeat the last token; never stored
+            const float* src = x + (size_t)tok * K + col;
+            if (vec_ok && col + 4 <= K) {
+                pf[i] = *reinterpret_cast<const float4*>(src);
+            } else {
+                pf[i].x = (col + 0 < K) ? src[0] : 0.0f;
+                pf[i].y = (col + 1 < K) ? src[1] : 0.0f;
+                pf[i].z = (col + 2 < K) ? src[2] : 0.0f;
+                pf[i].w = (col + 3 < K) ? src[3] : 0.0f;
+            }
+        }
+    };
+    float4 pf[PASSES];
+    if (blockIdx.x < total_tiles) fetch(pf, blockIdx.x);
+
+    for (uint32_t tile_id = blockIdx.x; tile_id < total_tiles; tile_id += gridDim.x) {
+    const uint32_t tok0 = (tile_id / tiles_cb) * TT;
+    const uint32_t cb0 = ((tile_id % tiles_cb) * S::WAVES + wave) * CBT;
+
+    // transpose through LDS: coalesced rows in, one row slice per lane out
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i)
+        *reinterpret_cast<float4*>(&tile[(fr0 + i * ROWS_PER_PASS) * PITCH + 4 * fq]) = pf[i];
+    __syncthreads();
     float xv[RF];
 #pragma unroll
     for (int i = 0; i < RF / 4; ++i) {
-        float4 t4 = *reinterpret_cast<const float4*>(&tile[threadIdx.x * PITCH + 4 * i]);
+        float4 t4 = *reinterpret_cast<const float4*>(&tile[lane * PITCH + wave * RF + 4 * i]);
         xv[4 * i + 0] = t4.x;
         xv[4 * i + 1] = t4.y;
         xv[4 * i + 2] = t4.z;
         xv[4 * i + 3] = t4.w;
     }
+    __syncthreads();  // every lane has its row slice: the tile may be overwritten
+    if (tile_id + gridDim.x < total_tiles) fetch(pf, tile_id + gridDim.x);
 
     // ---- distance + hysteresis scan, centroid order, one codebook after the other ----------
     constexpr int OUT_BITS = CBT * IDX_BITS;
@@ -91,13 +190,70 @@ __global__ __launch_bounds__(CCS_THREADS) void ccs_kernel(const float* __restric
 #pragma unroll
     for (int i = 0; i < OUT_WORDS; ++i) packed[i] = 0;
 
+    // Fast-form operands of one codebook: lane 16r+j holds (-2 c_0 .. -2 c_{v-1}, |c|^2) of centroid
+    // 16*grp+j, and a row_newbcast:j DPP operand hands that to all 16 lanes of the row.
+    const uint32_t groups = (C + 15) / 16;
+    auto load_aux = [&](float (&am)[V + 1], uint32_t cb, uint32_t grp) {
+        const uint32_t cbc = cb < CB ? cb : CB - 1;  // padded codebooks: any valid address
+        const float* __restrict__ ap = aux + ((size_t)cbc * (V + 1) * groups + grp) * 16 + (lane & 15);
 #pragma unroll
-    for (int cbl = 0; cbl < CBT; ++cbl) {
+        for (int t = 0; t <= V; ++t) am[t] = ap[(size_t)t * (16 * groups)];
+    };
+    constexpr bool PREFETCH = FAST && IDX_BITS == 4;  // C <= 16: one group per codebook
+    float am_ring[2][V + 1];
+    if constexpr (PREFETCH) load_aux(am_ring[0], cb0, 0);
+
+    static_for<CBT>([&](auto cbl_c) {
+        constexpr int cbl = decltype(cbl_c)::value;
         const uint32_t cb = cb0 + cbl;
         uint32_t bi = 0;
-        if (cb < CB) {  // wave-uniform
+        bool exact = (cb < CB);  // wave-uniform
+        if constexpr (PREFETCH && cbl + 1 < CBT) load_aux(am_ring[(cbl + 1) & 1], cb + 1, 0);
+        if (FAST && cb < CB) {
+            constexpr uint32_t ID_MASK = (1u << IDX_BITS) - 1u;
+            float xx = xv[cbl * V] * xv[cbl * V];
+#pragma unroll
+            for (int t = 1; t < V; ++t) xx = fmaf(xv[cbl * V + t], xv[cbl * V + t], xx);
+            float m1 = __builtin_inff(), m2 = __builtin_inff();
+            auto scan16 = [&](const float (&am)[V + 1], uint32_t c0) {
+                static_for<16>([&](auto jc) {
+                    constexpr int J = decltype(jc)::value;
+                    float sc;
+                    asm("v_add_f32_dpp %0, %1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf"
+                        : "=v"(sc) : "v"(am[V]), "v"(xx), "n"(J));
+#pragma unroll
+                    for (int t = 0; t < V; ++t)
+                        asm("v_fmac_f32_dpp %0, %1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf"
+                            : "+v"(sc) : "v"(am[t]), "v"(xv[cbl * V + t]), "n"(J));
+                    const uint32_t id = (IDX_BITS == 4) ? (uint32_t)J : (c0 | (uint32_t)J);
+                    const float key = __uint_as_float((__float_as_uint(sc) & ~ID_MASK) | id);
+                    m2 = __builtin_amdgcn_fmed3f(m1, m2, key);
+                    // plain v_min_f32: fminf() would first canonicalise the bit-cast key (one more op)
+                    asm("v_min_f32_e32 %0, %1, %2" : "=v"(m1) : "v"(m1), "v"(key));
+                });
+            };
+            if constexpr (PREFETCH) {
+                scan16(am_ring[cbl & 1], 0);
+            } else {
+                for (uint32_t grp = 0; grp < groups; ++grp) {
+                    float am[V + 1];
+                    load_aux(am, cb, grp);
+                    scan16(am, 16 * grp);
+                }
+            }
+            bi = __float_as_uint(m1) & ID_MASK;
+            const float mag = xx + cnmax[cb];
+            constexpr float A = 3.0f * (5 * V + 5) * 5.9604645e-8f;          // 3 (5v+5) u
+            constexpr float B = (float)(1u << IDX_BITS) * 2.3841858e-7f * 2;  // 2 * 2^(IDX_BITS-22)
+            const float thr = fmaf(A * 2.0f, mag, fmaf(B, fabsf(m2), 1.001e-6f));
+            // NaN anywhere makes a compare false, which counts as "not safe"
+            const bool safe = ((m2 - m1) > thr) && (mag < 1e36f);
+            exact = __builtin_amdgcn_ballot_w64(!safe) != 0;
+        }
+        if (exact) {
             const float* __restrict__ cp = cent + (size_t)cb * C * V;
             float best = 0.0f;
+            bi = 0;
 #pragma unroll 4
             for (uint32_t c = 0; c < C; ++c) {
                 // d = ((0 + d0*d0) + d1*d1) + ... ; 0.0f + p == p exactly for every p >= 0
@@ -115,11 +271,11 @@ __global__ __launch_bounds__(CCS_THREADS) void ccs_kernel(const float* __restric
         }
         constexpr int per_word = 32 / IDX_BITS;
         packed[cbl / per_word] |= bi << (IDX_BITS * (cbl % per_word));
-    }
+    });
 
     // ---- packed store -----------------------------------------------------------------------
-    const uint32_t tok = tok0 + threadIdx.x;
-    if (tok < N) {
+    const uint32_t tok = tok0 + lane;
+    if (tok < N && cb0 < CB_pad) {
         uint8_t* dst = idx + (size_t)tok * idx_row_bytes + (size_t)cb0 * IDX_BITS / 8;
         if constexpr (OUT_BITS >= 128) {
             *reinterpret_cast<uint4*>(dst) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
@@ -134,6 +290,7 @@ __global__ __launch_bounds__(CCS_THREADS) void ccs_kernel(const float* __restric
             *dst = (uint8_t)packed[0];
         }
     }
+    }  // tiles
 }
 
 // Generic sub-vector length (any v): one lane per (token, codebook), operands straight from
@@ -218,10 +375,27 @@ template <int V, int IDX_BITS>
 int launch_ccs_t(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_cent, uint8_t* d_idx, uint32_t n)
 {
     using S = CcsShape<V>;
-    dim3 grid((n + CCS_THREADS - 1) / CCS_THREADS, g.CB_pad / S::CBT);
+    const uint32_t cb_per_tile = S::WAVES * S::CBT;
+    const uint32_t tiles_cb = (g.CB_pad + cb_per_tile - 1) / cb_per_tile;
+    const uint64_t total64 = (uint64_t)((n + S::TILE_TOKENS - 1) / S::TILE_TOKENS) * tiles_cb;
+    if (total64 > 0xFFFFFFFFull) return set_error(ctx, PIMDL_ERR_INVALID, "ccs: too many tiles");
+    const uint32_t total = (uint32_t)total64;
+    // persistent grid: as many workgroups as stay resident (LDS bound, at most 4 per CU)
+    const uint32_t lds = S::LDS_BYTES;
+    uint32_t per_cu = (uint32_t)(160 * 1024 / lds);
+    if (per_cu > 4) per_cu = 4;
+    if (per_cu < 1) per_cu = 1;
+    const uint32_t slots = (uint32_t)ctx->prop.multiProcessorCount * per_cu;
+    dim3 grid(total < slots ? total : slots);
     const int vec_ok = (g.K % 4 == 0) && ((reinterpret_cast<uintptr_t>(d_x) & 15) == 0);
-    hipLaunchKernelGGL((ccs_kernel<V, IDX_BITS>), grid, dim3(CCS_THREADS), 0, ctx->stream, d_x, d_cent, d_idx, n,
-                       g.K, g.CB, g.C, g.idx_row_bytes, vec_ok);
+    const float* aux = d_cent + (size_t)g.CB * g.C * g.v;
+    const float* cnmax = aux + ccs_aux_floats(g);
+    if (ccs_exact_only())
+        hipLaunchKernelGGL((ccs_kernel<V, IDX_BITS, false>), grid, dim3(CCS_THREADS), 0, ctx->stream, d_x, d_cent,
+                           aux, cnmax, d_idx, n, g.K, g.CB, g.C, g.idx_row_bytes, vec_ok, g.CB_pad, tiles_cb, total);
+    else
+        hipLaunchKernelGGL((ccs_kernel<V, IDX_BITS, true>), grid, dim3(CCS_THREADS), 0, ctx->stream, d_x, d_cent,
+                           aux, cnmax, d_idx, n, g.K, g.CB, g.C, g.idx_row_bytes, vec_ok, g.CB_pad, tiles_cb, total);
     return hip_check(ctx, hipGetLastError(), "ccs_kernel launch");
 }
 
@@ -246,14 +420,39 @@ int launch_ccs_bits(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d
 
 }  // namespace
 
+// PIMDL_CCS_EXACT=1 in the environment switches the two-speed search off (every pair takes the
+// reference's scan); the results are the same by construction, so this is a debugging aid only.
+bool ccs_exact_only()
+{
+    static const bool v = [] {
+        const char* e = getenv("PIMDL_CCS_EXACT");
+        return e && e[0] == '1';
+    }();
+    return v;
+}
+
+size_t ccs_centroid_bytes(const AmmGeom& g)
+{
+    return ((size_t)g.CB * g.C * g.v + ccs_aux_floats(g) + g.CB) * sizeof(float);
+}
+
+int launch_ccs_prep(Ctx* ctx, const AmmGeom& g, float* d_cent)
+{
+    float* aux = d_cent + (size_t)g.CB * g.C * g.v;
+    float* cnmax = aux + ccs_aux_floats(g);
+    hipLaunchKernelGGL(ccs_prep_kernel, dim3(g.CB), dim3(64), 0, ctx->stream,
+                       d_cent, aux, cnmax, g.C, g.v);
+    return hip_check(ctx, hipGetLastError(), "ccs_prep_kernel launch");
+}
+
 uint32_t ccs_cb_per_wg(uint32_t v)
 {
     switch (v) {
-        case 2: return CcsShape<2>::CBT;
-        case 4: return CcsShape<4>::CBT;
-        case 8: return CcsShape<8>::CBT;
-        case 16: return CcsShape<16>::CBT;
-        case 32: return CcsShape<32>::CBT;
+        case 2: return CcsShape<2>::WAVES * CcsShape<2>::CBT;
+        case 4: return CcsShape<4>::WAVES * CcsShape<4>::CBT;
+        case 8: return CcsShape<8>::WAVES * CcsShape<8>::CBT;
+        case 16: return CcsShape<16>::WAVES * CcsShape<16>::CBT;
+        case 32: return CcsShape<32>::WAVES * CcsShape<32>::CBT;
         default: return 0;
     }
 }

@@ -614,7 +614,7 @@ bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::s
     g->M_pad = (M + g->col_block - 1) / g->col_block * g->col_block;
     g->ccs_cb_per_wg = ccs_cb_per_wg(v);
     g->ccs_row_floats = g->ccs_cb_per_wg * v;
-    g->ccs_lds_bytes = g->ccs_cb_per_wg ? 256 * (g->ccs_row_floats + 4) * 4 : 0;
+    g->ccs_lds_bytes = g->ccs_cb_per_wg ? 64 * (g->ccs_row_floats + 4) * 4 : 0;
     return true;
 }
 

@@ -267,11 +267,12 @@ int pimdl_amm_create(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const float* ce
     if (i8) retile_lut(reinterpret_cast<const int8_t*>(lut), reinterpret_cast<int8_t*>(tiled.data()), g, row_elems);
     else retile_lut(reinterpret_cast<const float*>(lut), reinterpret_cast<float*>(tiled.data()), g, row_elems);
 
-    rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&a->d_centroids), cent_bytes), "hipMalloc(centroids)");
+    rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&a->d_centroids), ccs_centroid_bytes(g)), "hipMalloc(centroids)");
     if (!rc) rc = hip_check(ctx, hipMalloc(&a->d_lut, a->lut_bytes), "hipMalloc(lut)");
     if (!rc) rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&a->d_bias), (size_t)g.M * sizeof(float)), "hipMalloc(bias)");
     if (!rc && i8) rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&a->d_scales), sizeof(float) * a->nscales), "hipMalloc(scales)");
     if (!rc) rc = hip_check(ctx, hipMemcpy(a->d_centroids, centroids, cent_bytes, hipMemcpyHostToDevice), "H2D centroids");
+    if (!rc) rc = launch_ccs_prep(ctx, g, a->d_centroids);
     if (!rc) rc = hip_check(ctx, hipMemcpy(a->d_lut, tiled.data(), a->lut_bytes, hipMemcpyHostToDevice), "H2D lut");
     if (!rc) {
         if (bias) rc = hip_check(ctx, hipMemcpy(a->d_bias, bias, (size_t)g.M * sizeof(float), hipMemcpyHostToDevice), "H2D bias");
@@ -418,8 +419,9 @@ int pimdl_index_calculation(pimdl_ctx* ctx, const float* in, const float* centro
     std::string why;
     if (!plan_geometry(d, ctx->prop.multiProcessorCount, &g, &why)) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_index_calculation: %s", why.c_str());
     const size_t cent_bytes = (size_t)g.CB * C * v * sizeof(float);
-    if ((rc = ensure(ctx, &ctx->d_cent, &ctx->cent_bytes, cent_bytes, "hipMalloc(centroid scratch)"))) return rc;
+    if ((rc = ensure(ctx, &ctx->d_cent, &ctx->cent_bytes, ccs_centroid_bytes(g), "hipMalloc(centroid scratch)"))) return rc;
     if ((rc = hip_check(ctx, hipMemcpyAsync(ctx->d_cent, centroids, cent_bytes, hipMemcpyHostToDevice, ctx->stream), "H2D centroids"))) return rc;
+    if ((rc = launch_ccs_prep(ctx, g, ctx->d_cent))) return rc;
     return index_calc_common(ctx, g, in, ctx->d_cent, n, idx_out, n_stile_size, cb_mtile_size);
 }
 
@@ -562,7 +564,7 @@ int pimdl_amm_get_geometry(const pimdl_amm* a, pimdl_amm_geometry* out)
     out->lds_bytes = g.gather_lds_bytes;
     out->tokens_per_wg = g.tokens_per_wg;
     out->gather_threads = g.gather_threads;
-    out->ccs_tokens_per_wg = 256;
+    out->ccs_tokens_per_wg = 64;
     out->ccs_cb_per_wg = g.ccs_cb_per_wg;
     out->ccs_threads = 256;
     out->ccs_lds_bytes = g.ccs_lds_bytes;

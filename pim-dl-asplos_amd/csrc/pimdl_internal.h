@@ -39,7 +39,7 @@ struct Amm {
     Ctx* ctx;
     pimdl_amm_desc desc;
     AmmGeom g;
-    float* d_centroids;  // [CB][C][v]
+    float* d_centroids;  // [CB][C][v], then the derived search data (ccs_centroid_bytes)
     void* d_lut;         // tiled
     size_t lut_bytes;
     float* d_scales;     // int8: scales
@@ -78,6 +78,11 @@ int hip_check(Ctx* ctx, hipError_t e, const char* what);
 // kernels (launchers validate nothing: callers have already checked shapes against AmmGeom)
 int launch_ccs(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_cent, uint8_t* d_idx,
                uint32_t n);
+// A centroid buffer holds the raw [CB][C][v] floats followed by data derived from them for the
+// search kernel; allocate ccs_centroid_bytes() and run launch_ccs_prep() after every upload.
+size_t ccs_centroid_bytes(const AmmGeom& g);
+int launch_ccs_prep(Ctx* ctx, const AmmGeom& g, float* d_cent);
+bool ccs_exact_only();
 int launch_gather(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_t* d_acc_or_null,
                   uint32_t n);
 int launch_unpack_idx(Ctx* ctx, const AmmGeom& g, const uint8_t* d_idx, uint16_t* d_idx16, uint32_t n,
