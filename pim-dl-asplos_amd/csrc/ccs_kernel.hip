@@ -64,6 +64,11 @@ inline size_t ccs_aux_floats(const AmmGeom& g)
     return (size_t)g.CB * (g.v + 1) * ((g.C + 15) / 16 * 16);
 }
 
+inline size_t ccs_aux_a_floats(const AmmGeom& g)
+{
+    return (size_t)(g.CB_pad / 2) * (g.v + 1) * 64 + g.CB_pad;  // A-operand images, padded cnmax
+}
+
 template <int N, typename F>
 __device__ __forceinline__ void static_for(F&& f)
 {
@@ -293,6 +298,297 @@ __global__ __launch_bounds__(CCS_THREADS) void ccs_kernel(const float* __restric
     }  // tiles
 }
 
+// =============================================================================================
+// Matrix-core search for C <= 16 (4-bit indices), v in {2, 4, 8}.
+//
+// The score  |c|^2 - 2 x.c  of 16 centroids x 2 codebooks x 32 tokens is one chain of v+1
+// v_mfma_f32_32x32x2_f32: the A operand holds, per codebook pair, a 32 x (2v+2) matrix whose row
+// for (codebook half h, centroid r) carries -2c in the v columns of its own codebook, zeros in the
+// other codebook's columns and |c|^2 in column 2v; the B operand holds the 2v activation values of
+// the pair and a 1.0 in row 2v.  Rows are ordered so that the result registers of lane (j, h)
+// are exactly the 16 scores of token j against codebook h of the pair:
+//     result register r of lane l = D[8*(r/4) + 4*(l/32) + r%4][l%32]   (hardware layout)
+//     => row i belongs to half h = (i/4)%2 and centroid r = i%4 + 4*(i/8).
+// The search is then lane-local: pack the centroid id into the low 4 mantissa bits, keep the two
+// smallest (v_and_or, v_med3, v_med3 per centroid) and apply the margin test described at the top
+// of this file.  (token, codebook) pairs that fail the test are replayed with the exact scan by
+// their own lane after the fast pass, from LDS copies of the activations and the raw centroids.
+//
+// A tile is 128 tokens x 16 codebooks.  Wave w owns codebook pairs 2w and 2w+1, whose A operands
+// stay in registers for the four 32-token groups of the tile; the next item's MFMA chain is issued
+// before the current item's scores are searched so the matrix pipe and the VALU overlap.
+// Workgroups are persistent and fetch the next tile's activations into registers meanwhile.
+//
+// Error bound of this form: |c|^2 carries <= v u CN, the MFMA chain rounds at most v+2 partial sums
+// each below 2(XX+CN): together with the reference chain's 2(v+2)u(XX+CN) that is below
+// (5v+8)u(XX+CN); the kernel uses twice that.
+// =============================================================================================
+template <int V>
+struct CcsMfmaShape {
+    static constexpr int TILE_TOKENS = 128;
+    static constexpr int CBW = 16;                         // codebooks per tile: 2 pairs per wave
+    static constexpr int TF = CBW * V;                     // floats per tile row
+    static constexpr int PITCH = TF + 4;                   // +16 B: odd number of 16-byte units
+    static constexpr int NQ = V + 1;                       // MFMAs (K = 2 each) per item
+    static constexpr int TG = TILE_TOKENS / 32;            // 32-token groups
+    static constexpr int ITEMS = 2 * TG;                   // (pair, token group) items per wave
+    static constexpr int X_FLOATS = TILE_TOKENS * PITCH;
+    static constexpr int CENT_FLOATS = CBW * 16 * V;       // raw centroids of the tile's codebooks
+    static constexpr int LDS_BYTES = (X_FLOATS + CENT_FLOATS) * 4 + TILE_TOKENS * (CBW / 2);
+};
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+// Plain hardware min/max on bit patterns that are already valid floats.  fminf()/fmaxf() would
+// first canonicalise operands that come from integer operations (one more VALU op each).
+__device__ __forceinline__ float vmin(float a, float b)
+{
+    float r;
+    asm("v_min_f32_e32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ __forceinline__ float vmax(float a, float b)
+{
+    float r;
+    asm("v_max_f32_e32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ __forceinline__ float vmin3(float a, float b, float c)
+{
+    float r;
+    asm("v_min3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+// Operands of the MFMA search behind the other derived data of a centroid buffer:
+//   aux_a     [CB_pad/2 pairs][v+1][64 lanes]  A-operand images
+//   cnmax_pad [CB_pad]                         cnmax, 0 for padded codebooks
+// A padded codebook scores r against centroid r, so it yields index 0 with a margin of 1.
+__global__ void ccs_prep_mfma_kernel(const float* __restrict__ cent, const float* __restrict__ cnmax,
+                                     float* __restrict__ aux_a, float* __restrict__ cnmax_pad, uint32_t CB,
+                                     uint32_t C, uint32_t v)
+{
+    const uint32_t pair = blockIdx.x, lane = threadIdx.x;
+    const uint32_t i = lane & 31, kh = lane >> 5;
+    const uint32_t h = (i >> 2) & 1, r = (i & 3) + 4 * (i >> 3);
+    const uint32_t cb = 2 * pair + h;
+    const bool real = (cb < CB) && (r < C);
+    const float* cp = cent + ((size_t)cb * C + r) * v;
+    float cn = (float)r;
+    if (real) {
+        cn = 0.0f;
+        for (uint32_t t = 0; t < v; ++t) cn = fmaf(cp[t], cp[t], cn);
+    } else if (cb < CB) {
+        cn = 3e38f;  // centroid ids past C never win
+    }
+    for (uint32_t q = 0; q <= v; ++q) {
+        const uint32_t k = 2 * q + kh;
+        float val = 0.0f;
+        if (k < 2 * v) {
+            if (real && k / v == h) val = -2.0f * cp[k % v];
+        } else if (k == 2 * v) {
+            val = cn;
+        }
+        aux_a[((size_t)pair * (v + 1) + q) * 64 + lane] = val;
+    }
+    if (lane < 2) {
+        const uint32_t c2 = 2 * pair + lane;
+        cnmax_pad[c2] = (c2 < CB) ? cnmax[c2] : 0.0f;
+    }
+}
+
+template <int V>
+__global__ __launch_bounds__(CCS_THREADS, 4) void ccs_mfma_kernel(const float* __restrict__ x,
+                                                                 const float* __restrict__ cent,
+                                                                 const float* __restrict__ aux_a,
+                                                                 const float* __restrict__ cnmax_pad,
+                                                                 uint8_t* __restrict__ idx, uint32_t N,
+                                                                 uint32_t K, uint32_t CB, uint32_t C,
+                                                                 uint32_t idx_row_bytes, int vec_ok,
+                                                                 uint32_t tiles_cb, uint32_t total_tiles)
+{
+    using S = CcsMfmaShape<V>;
+    constexpr int TF = S::TF, PITCH = S::PITCH, TT = S::TILE_TOKENS, NQ = S::NQ, CBW = S::CBW, TG = S::TG;
+    constexpr int ITEMS = S::ITEMS;
+    __shared__ __attribute__((aligned(16))) float tile[S::X_FLOATS];
+    __shared__ __attribute__((aligned(16))) float cst[S::CENT_FLOATS];
+    __shared__ __attribute__((aligned(16))) uint8_t ist[TT * (CBW / 2)];
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t j = lane & 31, h = lane >> 5;  // token within a group, codebook of the pair
+
+    constexpr int F4_PER_ROW = TF / 4;
+    constexpr int ROWS_PER_PASS = CCS_THREADS / F4_PER_ROW;
+    constexpr int PASSES = TT / ROWS_PER_PASS;
+    static_assert(CCS_THREADS % F4_PER_ROW == 0 && TT % ROWS_PER_PASS == 0, "tile shape");
+    const uint32_t fq = threadIdx.x % F4_PER_ROW;
+    const uint32_t fr0 = threadIdx.x / F4_PER_ROW;
+    auto fetch = [&](float4 (&pf)[PASSES], uint32_t tile_id) {
+        const uint32_t t_tok0 = (tile_id / tiles_cb) * TT;
+        const uint32_t col = (tile_id % tiles_cb) * TF + 4 * fq;
+#pragma unroll
+        for (int i = 0; i < PASSES; ++i) {
+            uint32_t tok = t_tok0 + fr0 + i * ROWS_PER_PASS;
+            if (tok >= N) tok = N - 1;  // rows past N repeat the last token; never stored
+            const float* src = x + (size_t)tok * K + col;
+            if (vec_ok && col + 4 <= K) {
+                pf[i] = *reinterpret_cast<const float4*>(src);
+            } else {
+                pf[i].x = (col + 0 < K) ? src[0] : 0.0f;
+                pf[i].y = (col + 1 < K) ? src[1] : 0.0f;
+                pf[i].z = (col + 2 < K) ? src[2] : 0.0f;
+                pf[i].w = (col + 3 < K) ? src[3] : 0.0f;
+            }
+        }
+    };
+    // operands of this lane inside the tile: row of token (32 tg + j), columns of pair (2 wave + pl)
+    const float* brow0 = tile + j * PITCH + 2 * wave * 2 * V;
+    const float b_last = (h == 0) ? 1.0f : 0.0f;
+
+    float4 pf[PASSES];
+    if (blockIdx.x < total_tiles) fetch(pf, blockIdx.x);
+
+    for (uint32_t tile_id = blockIdx.x; tile_id < total_tiles; tile_id += gridDim.x) {
+        const uint32_t tok0 = (tile_id / tiles_cb) * TT;
+        const uint32_t tcb = tile_id % tiles_cb;          // codebooks 16 tcb .. 16 tcb + 15
+        const uint32_t pair0 = tcb * (CBW / 2) + 2 * wave;  // first of this wave's two pairs
+
+        float aq[2][NQ];
+#pragma unroll
+        for (int pl = 0; pl < 2; ++pl)
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) aq[pl][q] = aux_a[((size_t)(pair0 + pl) * NQ + q) * 64 + lane];
+        // every global load the search needs is issued here, ahead of the next tile's prefetch:
+        // loads complete in order, so a later load would have to wait for the prefetch from HBM
+        float cmax[2];
+#pragma unroll
+        for (int pl = 0; pl < 2; ++pl) cmax[pl] = cnmax_pad[2 * (pair0 + pl) + h];
+        // raw centroids of the tile's codebooks, only read by exact replays
+        const uint32_t cb_here = (CB - tcb * CBW < (uint32_t)CBW) ? CB - tcb * CBW : (uint32_t)CBW;
+        const uint32_t cent_fl = cb_here * C * V;
+        const float* csrc = cent + (size_t)tcb * CBW * C * V;  // 16-byte aligned: CBW * V * 4 bytes per c
+#pragma unroll
+        for (int i = 0; i < PASSES; ++i)
+            *reinterpret_cast<float4*>(&tile[(fr0 + i * ROWS_PER_PASS) * PITCH + 4 * fq]) = pf[i];
+        for (uint32_t i = threadIdx.x; i < cent_fl / 4; i += CCS_THREADS)
+            reinterpret_cast<float4*>(cst)[i] = reinterpret_cast<const float4*>(csrc)[i];
+        if (threadIdx.x < cent_fl % 4) cst[cent_fl - 1 - threadIdx.x] = csrc[cent_fl - 1 - threadIdx.x];
+        __syncthreads();
+        if (tile_id + gridDim.x < total_tiles) fetch(pf, tile_id + gridDim.x);
+
+        auto scores = [&](floatx16& acc, int it) {
+            const int pl = it / TG, tg = it % TG;
+            const float* brow = brow0 + tg * 32 * PITCH + pl * 2 * V;
+            acc = floatx16(0.0f);
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) {
+                const float b = (q < V) ? brow[2 * q + h] : b_last;
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(aq[pl][q], b, acc, 0, 0, 0);
+            }
+        };
+
+        // words[tg / 2], 16 bits per token group: nibble of (pair pl, half h) at bit 8 pl + 4 h
+        uint32_t words[TG / 2];
+#pragma unroll
+        for (int i = 0; i < TG / 2; ++i) words[i] = 0;
+        uint32_t need = 0;  // bit it: item it must be replayed exactly by this lane
+
+        floatx16 acc_cur, acc_nxt;
+        scores(acc_cur, 0);
+        static_for<ITEMS>([&](auto itc) {
+            constexpr int it = decltype(itc)::value;
+            constexpr int pl = it / TG, tg = it % TG;
+            if constexpr (it + 1 < ITEMS) scores(acc_nxt, it + 1);
+            // |x|^2 of this lane's own codebook, for the error bound
+            const float* xo = brow0 + tg * 32 * PITCH + pl * 2 * V + V * h;
+            float xx = xo[0] * xo[0];
+#pragma unroll
+            for (int t = 1; t < V; ++t) xx = fmaf(xo[t], xo[t], xx);
+            // smallest (m1) and second smallest (m2) of the 16 id-tagged scores, 36 VALU operations:
+            // five triples give (min3, med3) each; the overall second smallest is the smaller of
+            // the second smallest of the six group minima and the smallest of the group medians.
+            float key[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                key[r] = __uint_as_float((__float_as_uint(acc_cur[r]) & ~15u) | (uint32_t)r);
+            float lo[5], md[5];
+#pragma unroll
+            for (int i = 0; i < 5; ++i) {
+                lo[i] = vmin3(key[3 * i], key[3 * i + 1], key[3 * i + 2]);
+                md[i] = __builtin_amdgcn_fmed3f(key[3 * i], key[3 * i + 1], key[3 * i + 2]);
+            }
+            const float a1 = vmin3(lo[0], lo[1], lo[2]), a2 = __builtin_amdgcn_fmed3f(lo[0], lo[1], lo[2]);
+            const float b1 = vmin3(lo[3], lo[4], key[15]), b2 = __builtin_amdgcn_fmed3f(lo[3], lo[4], key[15]);
+            const float m1 = vmin(a1, b1);
+            const float m2 = vmin3(vmin3(md[0], md[1], md[2]), vmin3(md[3], md[4], vmax(a1, b1)), vmin(a2, b2));
+            const uint32_t bi = __float_as_uint(m1) & 15u;
+            const float mag = xx + cmax[pl];
+            constexpr float A2 = 2.0f * 2.0f * (5 * V + 8) * 5.9604645e-8f;  // 2 * [2 (5v+8) u]
+            constexpr float B2 = 2.0f * 16.0f * 2.3841858e-7f;               // 2 * 2^(4-22)
+            const float thr = fmaf(A2, mag, fmaf(B2, fabsf(m2), 1.001e-6f));
+            // NaN anywhere makes a compare false, which counts as "not safe"
+            const bool safe = ((m2 - m1) > thr) && (mag < 1e36f);
+            need |= (safe ? 0u : 1u) << it;
+            words[tg / 2] |= bi << (16 * (tg % 2) + 8 * pl + 4 * h);
+            if constexpr (it + 1 < ITEMS) acc_cur = acc_nxt;
+        });
+
+        // ---- exact replay of the items that failed the margin test (rare, lane-divergent) -------
+        if (__builtin_amdgcn_ballot_w64(need != 0) != 0) {
+            // kept rolled on purpose: the replay is rare and must not cost the fast path registers
+#pragma nounroll
+            for (int it = 0; it < ITEMS; ++it) {
+                if (!((need >> it) & 1u)) continue;
+                const int pl = it / TG, tg = it % TG;
+                const uint32_t cbl = 2 * (2 * wave + pl) + h;
+                uint32_t bi = 0;
+                if (tcb * CBW + cbl < CB) {
+                    const float* xo = brow0 + tg * 32 * PITCH + pl * 2 * V + V * h;
+                    const float* cp = cst + cbl * C * V;
+                    float best = 0.0f;
+#pragma nounroll
+                    for (uint32_t c = 0; c < C; ++c) {
+                        float diff = __fsub_rn(xo[0], cp[c * V + 0]);
+                        float d = __fmul_rn(diff, diff);
+#pragma unroll
+                        for (int t = 1; t < V; ++t) {
+                            diff = __fsub_rn(xo[t], cp[c * V + t]);
+                            d = __fadd_rn(d, __fmul_rn(diff, diff));
+                        }
+                        const bool take = (c == 0) || (__fsub_rn(best, d) > 1e-6f);
+                        best = take ? d : best;
+                        bi = take ? c : bi;
+                    }
+                }
+                const uint32_t sh = 16 * (tg % 2) + 8 * pl + 4 * h;
+                uint32_t w = words[0];
+#pragma unroll
+                for (int i = 1; i < TG / 2; ++i) w = (tg / 2 == i) ? words[i] : w;
+                w = (w & ~(15u << sh)) | (bi << sh);
+#pragma unroll
+                for (int i = 0; i < TG / 2; ++i) words[i] = (tg / 2 == i) ? w : words[i];
+            }
+        }
+
+        // ---- merge the two codebooks of each pair (lanes l and l+32), gather the tile's index
+        //      bytes in LDS, store 8 bytes per token ------------------------------------------------
+#pragma unroll
+        for (int i = 0; i < TG / 2; ++i) words[i] |= __shfl_xor(words[i], 32);
+        if (h == 0) {
+#pragma unroll
+            for (int tg = 0; tg < TG; ++tg)
+                *reinterpret_cast<uint16_t*>(&ist[(32 * tg + j) * (CBW / 2) + 2 * wave]) =
+                    (uint16_t)(words[tg / 2] >> (16 * (tg % 2)));
+        }
+        __syncthreads();  // index bytes complete; every wave is done with the activation tile
+        if (threadIdx.x < TT) {
+            const uint32_t tok = tok0 + threadIdx.x;
+            if (tok < N)
+                *reinterpret_cast<uint2*>(idx + (size_t)tok * idx_row_bytes + tcb * (CBW / 2)) =
+                    *reinterpret_cast<const uint2*>(&ist[threadIdx.x * (CBW / 2)]);
+        }
+    }
+}
+
 // Generic sub-vector length (any v): one lane per (token, codebook), operands straight from
 // global memory.  Correct for every shape; only used where no specialisation exists.
 template <int IDX_BITS>
@@ -399,9 +695,44 @@ int launch_ccs_t(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_ce
     return hip_check(ctx, hipGetLastError(), "ccs_kernel launch");
 }
 
+template <int V>
+int launch_ccs_mfma(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_cent, uint8_t* d_idx, uint32_t n)
+{
+    using S = CcsMfmaShape<V>;
+    const uint32_t tiles_cb = g.CB_pad / S::CBW;  // CB_pad is a multiple of 32
+    const uint64_t total64 = (uint64_t)((n + S::TILE_TOKENS - 1) / S::TILE_TOKENS) * tiles_cb;
+    if (total64 > 0xFFFFFFFFull) return set_error(ctx, PIMDL_ERR_INVALID, "ccs: too many tiles");
+    const uint32_t total = (uint32_t)total64;
+    // persistent grid: exactly the workgroups that are resident at once
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, ccs_mfma_kernel<V>, CCS_THREADS, 0) != hipSuccess ||
+        per_cu < 1) {
+        (void)hipGetLastError();
+        per_cu = 1;
+    }
+    const uint32_t slots = (uint32_t)ctx->prop.multiProcessorCount * (uint32_t)per_cu;
+    dim3 grid(total < slots ? total : slots);
+    const int vec_ok = (g.K % 4 == 0) && ((reinterpret_cast<uintptr_t>(d_x) & 15) == 0);
+    const float* aux = d_cent + (size_t)g.CB * g.C * g.v;
+    const float* cnmax = aux + ccs_aux_floats(g);
+    const float* aux_a = cnmax + g.CB;
+    const float* cnmax_pad = aux_a + (size_t)(g.CB_pad / 2) * (g.v + 1) * 64;
+    hipLaunchKernelGGL((ccs_mfma_kernel<V>), grid, dim3(CCS_THREADS), 0, ctx->stream, d_x, d_cent, aux_a, cnmax_pad,
+                       d_idx, n, g.K, g.CB, g.C, g.idx_row_bytes, vec_ok, tiles_cb, total);
+    return hip_check(ctx, hipGetLastError(), "ccs_mfma_kernel launch");
+}
+
 template <int IDX_BITS>
 int launch_ccs_bits(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_cent, uint8_t* d_idx, uint32_t n)
 {
+    if (IDX_BITS == 4 && !ccs_exact_only()) {
+        switch (g.v) {
+            case 2: return launch_ccs_mfma<2>(ctx, g, d_x, d_cent, d_idx, n);
+            case 4: return launch_ccs_mfma<4>(ctx, g, d_x, d_cent, d_idx, n);
+            case 8: return launch_ccs_mfma<8>(ctx, g, d_x, d_cent, d_idx, n);
+            default: break;
+        }
+    }
     switch (g.v) {
         case 2: return launch_ccs_t<2, IDX_BITS>(ctx, g, d_x, d_cent, d_idx, n);
         case 4: return launch_ccs_t<4, IDX_BITS>(ctx, g, d_x, d_cent, d_idx, n);
@@ -433,7 +764,7 @@ bool ccs_exact_only()
 
 size_t ccs_centroid_bytes(const AmmGeom& g)
 {
-    return ((size_t)g.CB * g.C * g.v + ccs_aux_floats(g) + g.CB) * sizeof(float);
+    return ((size_t)g.CB * g.C * g.v + ccs_aux_floats(g) + g.CB + ccs_aux_a_floats(g)) * sizeof(float);
 }
 
 int launch_ccs_prep(Ctx* ctx, const AmmGeom& g, float* d_cent)
@@ -442,7 +773,12 @@ int launch_ccs_prep(Ctx* ctx, const AmmGeom& g, float* d_cent)
     float* cnmax = aux + ccs_aux_floats(g);
     hipLaunchKernelGGL(ccs_prep_kernel, dim3(g.CB), dim3(64), 0, ctx->stream,
                        d_cent, aux, cnmax, g.C, g.v);
-    return hip_check(ctx, hipGetLastError(), "ccs_prep_kernel launch");
+    int rc = hip_check(ctx, hipGetLastError(), "ccs_prep_kernel launch");
+    if (rc) return rc;
+    float* aux_a = cnmax + g.CB;
+    hipLaunchKernelGGL(ccs_prep_mfma_kernel, dim3(g.CB_pad / 2), dim3(64), 0, ctx->stream, d_cent, cnmax, aux_a,
+                       aux_a + (size_t)(g.CB_pad / 2) * (g.v + 1) * 64, g.CB, g.C, g.v);
+    return hip_check(ctx, hipGetLastError(), "ccs_prep_mfma_kernel launch");
 }
 
 uint32_t ccs_cb_per_wg(uint32_t v)
