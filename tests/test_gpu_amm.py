@@ -205,3 +205,67 @@ def test_error_paths(ctx):
     assert e.value.code == -1
     assert amm.run(np.zeros((0, 16), np.float32)).shape == (0, 8)  # empty batch is a no-op
     amm.close()
+
+
+# ---- the two-speed search: fast scores + margin test, exact replay on near ties -----------------
+
+@pytest.mark.parametrize("v,C", [(2, 16), (4, 16), (8, 16), (4, 7), (16, 16), (4, 32), (2, 64)])
+def test_search_with_exact_ties_and_degenerate_inputs(ctx, v, C):
+    """Duplicate centroids (margin 0), all-zero rows, inputs equal to a centroid, tiny and huge
+    magnitudes: every pair must come out as the reference's scan says, whichever path took it."""
+    rng = np.random.default_rng(1000 + 10 * v + C)
+    N, CB = 389, 37
+    cent = rng.standard_normal((CB, C, v)).astype(np.float32)
+    cent[::3, C // 2] = cent[::3, 0]                   # exact duplicates: first index must win
+    cent[1::5] *= np.float32(1e-3)                     # a codebook of tiny centroids
+    cent[2::7] *= np.float32(1e4)                      # and one of huge ones
+    x = rng.standard_normal((N, CB, v)).astype(np.float32)
+    x[::4] = 0.0
+    pick = rng.integers(0, C, (N, CB))
+    on = rng.random((N, CB)) < 0.3
+    x[on] = cent[np.nonzero(on)[1], pick[on]]          # exactly on a centroid
+    x[5::11] *= np.float32(1e5)
+    x = x.reshape(N, CB * v)
+    want = oracle.index_calculation(x, cent, v, threads=THREADS)
+    amm = ctx.amm(cent, np.zeros((CB, C, 4), np.int8), np.float32(1.0), None, max_n=N)
+    got = amm.index_calculation(x)
+    assert np.array_equal(got, want), f"{(got != want).sum()} of {got.size} differ"
+    amm.close()
+
+
+@pytest.mark.parametrize("v,C", [(4, 16), (2, 16), (8, 16), (4, 32)])
+def test_search_with_non_finite_values(ctx, v, C):
+    """NaN / Inf / near-overflow values in activations and centroids take the exact path and match
+    the reference's compare semantics (a NaN distance never replaces the running best)."""
+    rng = np.random.default_rng(2000 + 10 * v + C)
+    N, CB = 300, 40
+    cent = rng.standard_normal((CB, C, v)).astype(np.float32)
+    cent[3, 2, 0] = np.nan
+    cent[5, 0, 1] = np.nan          # NaN in centroid 0: the scan keeps index 0
+    cent[7, 4, 0] = np.inf
+    cent[9, 1, :] = 3e19            # |c|^2 overflows fp32
+    cent[11, 6, 0] = -np.inf
+    x = rng.standard_normal((N, CB * v)).astype(np.float32)
+    x[1, :] = np.nan
+    x[2, 5] = np.inf
+    x[3, 7] = -np.inf
+    x[4, :] = 2e19
+    x[6, 3] = 3e38
+    with np.errstate(all="ignore"):
+        want = oracle.index_calculation(x, cent, v, threads=THREADS)
+    amm = ctx.amm(cent, np.zeros((CB, C, 4), np.int8), np.float32(1.0), None, max_n=N)
+    got = amm.index_calculation(x)
+    assert np.array_equal(got, want), f"{(got != want).sum()} of {got.size} differ"
+    amm.close()
+
+
+def test_search_at_full_ffn2_shape(ctx):
+    """N=8192, K=3072, v=4, 16 centroids: every index of the headline shape against the oracle,
+    once with N(0,1) data and once with the reference driver's ranges."""
+    for dist in ("normal", "ref"):
+        x, cent, _, _ = make_case(77, 8192, 3072, 4, 16, 4, "i8", dist)
+        want = oracle.index_calculation(x, cent, 4, threads=THREADS)
+        amm = ctx.amm(cent, np.zeros((768, 16, 4), np.int8), np.float32(1.0), None, max_n=8192)
+        got = amm.index_calculation(x)
+        assert np.array_equal(got, want), f"{dist}: {(got != want).sum()} of {got.size} differ"
+        amm.close()

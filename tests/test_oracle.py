@@ -72,6 +72,28 @@ def _one_subvector(dists):
     return x, cent, (roots * roots).astype(np.float32)
 
 
+@pytest.mark.skipif(not oracle.have_ref(), reason="oracle/_ref not built (needs the reference tree)")
+def test_index_matches_reference_live_on_non_finite_values():
+    """NaN / Inf / overflowing values: the restatement must keep the reference's compare semantics
+    (`best - d > 1e-6` is false for NaN, so a NaN never replaces the running best)."""
+    rng = np.random.default_rng(7)
+    N, CB, C, v = 64, 24, 16, 4
+    cent = rng.standard_normal((CB, C, v)).astype(np.float32)
+    cent[3, 2, 0] = np.nan
+    cent[5, 0, 1] = np.nan
+    cent[7, 4, 0] = np.inf
+    cent[9, 1, :] = 3e19
+    x = rng.standard_normal((N, CB * v)).astype(np.float32)
+    x[1, :] = np.nan
+    x[2, 5] = np.inf
+    x[4, :] = 2e19
+    with np.errstate(all="ignore"):
+        got = oracle.index_calculation(x, cent, v, threads=2)
+        want = oracle.ref_index_calculation(x, cent, v, threads=2)
+    assert np.array_equal(got, want)
+    assert (got[:, 5] == 0).all()  # NaN in centroid 0 pins the scan at index 0
+
+
 def test_scan_hysteresis_closed_forms():
     # equal to centroid j => j
     rng = np.random.default_rng(1)
