@@ -21,6 +21,15 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0                     # MI355X HBM3E
+# HBM bytes per launch of the gather kernels at this workload, from two rocprofv3 --pmc runs of this
+# script (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch).  FETCH_SIZE is scaled by 2.0 and
+# WRITE_SIZE by 1.0: the factors a streaming kernel of known size gives for the same counters on
+# this part.  Summary: profiles/bench_ffn_pair_hbm_traffic.txt.  Keyed by (K, M).
+MEASURED_GATHER_TRAFFIC = {
+    (768, 3072): {"fetch_kib": 37581.4, "write_kib": 101973.0},
+    (3072, 768): {"fetch_kib": 39011.9, "write_kib": 24748.0},
+}
+FETCH_SCALE, WRITE_SCALE = 2.0, 1.0
 LDS_PEAK_GBPS = 256 * 256 * 2.4            # 256 CUs x 256 B/clk (ds_read_b128) x 2.4 GHz = 157286 GB/s
 
 
@@ -168,11 +177,15 @@ def main():
     K, M = dom["K"], dom["M"]
     ab = algorithmic_bytes(N, K, v, C, M)
     _, lds_measured = ctx.diag_bandwidth(copy=False, lds=True)
+    mt = MEASURED_GATHER_TRAFFIC.get((K, M)) if N == 8192 else None
+    traffic = (mt["fetch_kib"] * FETCH_SCALE + mt["write_kib"] * WRITE_SCALE) * 1024.0 if mt else None
     roofline = {
         "kernel": f"gather_i8_kernel ({dom['name']}: K={K} M={M})",
         "bound": "lds", "achieved": dom["gather_lds_gbps"], "peak": LDS_PEAK_GBPS, "unit": "GB/s",
         "frac": dom["gather_lds_frac"],
-        "traffic": None,
+        "traffic": traffic,
+        "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this script, scaled x2.0 / x1.0 "
+                          "(copy-kernel calibration); recorded constant, not collected in this run",
         "algorithmic_bytes_per_launch": ab["gather_lds"],
         "avg_launch_ms": dom["gather_ms"],
         "lds_peak_measured_gbps": lds_measured,
