@@ -35,6 +35,8 @@
 //
 // fp32 kernel.  Same staging; one lane owns one token and adds rows in ascending codebook order
 // (bit-identical to a sequential CPU sum).
+#include <stdlib.h>
+
 #include <type_traits>
 
 #include "pimdl_internal.h"
@@ -77,6 +79,11 @@ template <int OFF>
 __device__ __forceinline__ void lds_read(v4i& slot, uint32_t addr)
 {
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(slot) : "v"(addr), "n"(OFF));
+}
+template <int OFF>
+__device__ __forceinline__ void lds_read32(uint32_t& dst, uint32_t addr)
+{
+    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
 }
 template <int OFF, int WAIT>
 __device__ __forceinline__ void mfma_then_read(v4i& acc, v4i& slot, const v4i& a, uint32_t addr)
@@ -394,6 +401,396 @@ __global__ __launch_bounds__(GATHER_THREADS, 4) void gather_i8_kernel(
     if (pending_epilogue) epilogue(epilogue_item);
 }
 
+
+// =============================================================================================
+// One-hot matrix-core gather for C <= 16 (int8 LUT, 4-bit indices).
+//
+// The byte-adder kernel above reads every gathered row piece from LDS once per token: N*CB*M
+// bytes, which ties it to LDS read bandwidth and leaves the matrix core waiting.  For C <= 16 the
+// same v_mfma_i32_16x16x64_i8 does the same amount of gathering per instruction (16 tokens x 16
+// columns x 4 codebooks) in the reference's own definition of the operator
+// (model-calibration/LUTNeuro/LUTLinear_t.py:78, bmm(one_hot, lut)):
+//     A[i][16 g + c] = lut[cb_g][c][column i]        (the 16 centroid rows of 4 codebooks)
+//     B[16 g + c][j] = (idx[token j][cb_g] == c)     (one-hot of token j's index)
+//     D[i][j] += sum over g of lut[cb_g][idx[j][cb_g]][i]
+// Both operands are now shared: one A operand serves every token of the tile, one B operand every
+// column, so a wave that keeps TM token groups x TN column groups of accumulators issues TM*TN
+// MFMAs per TM+TN LDS reads (0.42 reads per MFMA at 4 x 6 instead of 1), and the kernel is bound by
+// the matrix core.  The sum is still an exact int32 sum of int8 entries.
+//
+// LUT layout for this kernel (HBM and LDS alike): [column tile][codebook][column][16 centroids],
+// so a lane's A operand is 16 consecutive bytes, lanes of a column group read consecutive 16-byte
+// units (no bank conflicts), and a slice of 16 codebooks is one contiguous block that goes from
+// L2 to LDS with global_load_lds (no registers, no ds_write).
+// The one-hot operand comes from a 256-byte table in LDS (entry c = 16 bytes with byte c set):
+// lanes with equal indices read the same address (broadcast), others hit different banks.
+//
+// A workgroup is four waves; wave w owns tokens 64 w .. 64 w + 63 of a 256-token tile (TM = 4)
+// and all 16*TN columns of the tile.  Workgroups are persistent over a flat (item, slice) stream,
+// double-buffered in LDS, one barrier per slice.
+// =============================================================================================
+constexpr int OH_WAVES = 4;
+constexpr int OH_THREADS = OH_WAVES * 64;
+constexpr int OH_TM = 4;                              // 16-token groups per wave
+constexpr int OH_TOK_ITEM = OH_WAVES * OH_TM * 16;    // 256 tokens per item
+
+// codebooks per slice (4 per MFMA K-step)
+constexpr int oh_slice_cbs(int) { return 16; }
+// LUT slice buffers in LDS (prefetch distance = buffers - 1); two workgroups must fit in a CU's LDS
+constexpr int oh_nbuf(int) { return 3; }
+// one-hot table + LUT slice buffers + index buffers
+constexpr int oh_lds_bytes(int tn)
+{
+    return 256 + oh_nbuf(tn) * oh_slice_cbs(tn) * 16 * tn * 16 + oh_nbuf(tn) * OH_TOK_ITEM * (oh_slice_cbs(tn) / 2);
+}
+
+// all operands of one K-step have landed; the registers pass through the asm so that no consumer
+// can be scheduled ahead of the wait
+template <int TN>
+__device__ __forceinline__ void oh_wait(v4i (&a)[TN], v4i (&b)[OH_TM])
+{
+    static_assert(OH_TM == 4, "operand list");
+    if constexpr (TN == 3)
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
+    else if constexpr (TN == 4)
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
+    else {
+        static_assert(TN == 6, "operand list");
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
+    }
+}
+
+// A workgroup is four waves; wave w owns tokens 64 w .. 64 w + 63 of a 256-token tile (TM = 4) and
+// all 16*TN columns of the tile; two workgroups per CU put two waves on every SIMD (one wave alone
+// can only issue an MFMA every ~30 cycles; two keep the matrix core at its ~21).  Smaller wave
+// tiles with more waves were slower: a K-step must hold enough MFMAs (TM*TN) to cover the LDS
+// latency of the next K-step's operands.
+template <int TN>
+__global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
+    const uint8_t* __restrict__ idx, const int8_t* __restrict__ lut, float* __restrict__ out,
+    int32_t* __restrict__ acc_out, uint32_t N, uint32_t M, uint32_t CB_pad, uint32_t idx_row_bytes,
+    uint32_t n_token_tiles, uint32_t n_items, Epilogue ep)
+{
+    constexpr int TM = OH_TM;
+    constexpr int WN = 16 * TN;                    // columns per item
+    constexpr int G = oh_slice_cbs(TN);            // codebooks per slice
+    constexpr int SLICE = G * WN * 16;             // bytes of one codebook slice
+    constexpr int KSTEPS = G / 4;
+    constexpr int IWORDS = G / 8;                  // 32-bit index words per token and slice
+    constexpr int NBLK = SLICE / 1024;             // 1 KB blocks (one copy instruction of a wave) per slice
+    constexpr int DMA_PER_WAVE = (NBLK + OH_WAVES - 1) / OH_WAVES;
+
+    // LDS: one-hot table (256 B) | NBUF LUT slice buffers | NIBUF index buffers
+    // (index words k+1 .. k+PD+1 are live while slice k is consumed; words k are in registers)
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    constexpr int NBUF = oh_nbuf(TN), NIBUF = NBUF;
+    constexpr int PD = NBUF - 1;  // prefetch distance of the LUT stream, in slices
+    constexpr uint32_t BUF0 = 256;  // the table sits at LDS offset 0: entry address = nibble * 16
+    constexpr uint32_t IBUF0 = BUF0 + NBUF * SLICE;
+    constexpr uint32_t IBYTES = OH_TOK_ITEM * (G / 2);        // index bytes of one slice
+    constexpr uint32_t IWAVE = 64 * (G / 2);                  // ... of one wave's 64 tokens
+    constexpr int IX_OPS = IWORDS;                            // 64 lanes x 4 B = 64 tokens x 1 word
+    constexpr int DMA_OPS = DMA_PER_WAVE + IX_OPS;            // memory operations per wave and slice
+
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: addresses below stay in SGPRs
+    const uint32_t j = lane & 15;  // column within a group (A operand) / token within a group (B operand)
+    const uint32_t g = lane >> 4;  // codebook of the K-step
+    if (blockIdx.x >= n_items) return;  // whole workgroup
+    const uint32_t nslices = CB_pad / G;
+    const uint32_t my_items = (n_items - blockIdx.x + gridDim.x - 1) / gridDim.x;
+    const uint32_t total = my_items * nslices;
+
+    if (threadIdx.x < 64) {  // entry e = 16 bytes, byte e is 1
+        const uint32_t e = threadIdx.x >> 2, w = threadIdx.x & 3;
+        reinterpret_cast<uint32_t*>(smem)[threadIdx.x] = ((e >> 2) == w) ? (1u << (8 * (e & 3))) : 0u;
+    }
+
+    // Everything comes in through global_load_lds, so the only memory-counter waits in the loop are
+    // the explicit ones.  Two independent stream positions step through the (item, slice) sequence:
+    // the LUT position runs PD slices ahead of the one being consumed, the index position PD+1
+    // (the index words of slice k+1 are unpacked while slice k is multiplied).
+    //   LUT:   wave w copies the 1 KB blocks w, w+8, .. of a slice; where the blocks do not divide
+    //          evenly a wave copies its first block twice, so that every wave issues the same
+    //          number of operations per slice (the waits below count them).
+    //   index: lane L of wave w copies index word i of token 64 w + L with its i-th operation,
+    //          into [wave][word][64 tokens]; only the wave itself reads them back.
+    // Addresses are kept as a wave-uniform 64-bit base (scalar registers) plus a 32-bit per-lane
+    // offset, the form the copy instructions take directly.
+    uint32_t lut_item = blockIdx.x, lut_s = 0, ix_item = blockIdx.x, ix_s = 0;
+    const int8_t* dma_base;   // uniform: start of the slice at the LUT stream position
+    const uint32_t dma_lane = wave * 1024 + lane * 16;
+    const uint8_t* ix_base;   // uniform: idx + byte offset of the slice inside a row
+    uint32_t ix_lane_off;     // per lane: token row offset (rows of one workgroup tile span < 4 GB: checked at launch)
+    auto locate_lut = [&]() {
+        dma_base = lut + (size_t)(lut_item / n_token_tiles) * CB_pad * (WN * 16);
+    };
+    auto locate_ix = [&]() {
+        uint32_t tok = (ix_item % n_token_tiles) * OH_TOK_ITEM + wave * 64 + lane;
+        if (tok >= N) tok = N - 1;  // clamp: results of such tokens are never stored
+        ix_base = idx;
+        ix_lane_off = tok * idx_row_bytes;
+    };
+    // real = false (past the end of the stream): the operation re-copies the first slice of the
+    // LUT into a buffer nobody reads any more, so that every slice issues the same number of
+    // operations and the waits can count them
+    auto lut_op = [&](uint32_t buf, bool real, auto uc) {
+        constexpr int u = decltype(uc)::value;
+        const uint32_t dst = BUF0 + buf * SLICE + wave * 1024;  // wave-uniform; lanes add 16*lane
+        const uint32_t off = (wave + OH_WAVES * u < NBLK) ? OH_WAVES * u * 1024 : 0;  // wave-uniform
+        const int8_t* src = (real ? dma_base : lut) + off;  // uniform
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + dma_lane),
+                                         (__attribute__((address_space(3))) void*)(smem + dst + off), 16, 0, 0);
+    };
+    auto lut_advance = [&]() {
+        dma_base += SLICE;
+        if (++lut_s == nslices) {
+            lut_s = 0;
+            lut_item += gridDim.x;
+            locate_lut();  // may point past the last item; never dereferenced then
+        }
+    };
+    auto stage_lut = [&](uint32_t buf) {
+        static_for<0, DMA_PER_WAVE>([&](auto uc) { lut_op(buf, true, uc); });
+        lut_advance();
+    };
+    // real = false: as above, into an index buffer nobody will unpack
+    auto ix_op = [&](uint32_t ibuf, bool real, auto ic) {
+        constexpr int i = decltype(ic)::value;
+        const uint32_t dst = IBUF0 + ibuf * IBYTES + wave * IWAVE;  // wave-uniform; lanes add 4*lane
+        const uint8_t* src = real ? ix_base + 4 * i : idx;  // uniform
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + (real ? ix_lane_off : 0u)),
+                                         (__attribute__((address_space(3))) void*)(smem + dst + 256 * i), 4, 0, 0);
+    };
+    auto ix_advance = [&]() {
+        ix_base += G / 2;
+        if (++ix_s == nslices) {
+            ix_s = 0;
+            ix_item += gridDim.x;
+            if (ix_item < n_items) locate_ix();
+        }
+    };
+    auto stage_ix = [&](uint32_t ibuf) {
+        static_for<0, IX_OPS>([&](auto ic) { ix_op(ibuf, true, ic); });
+        ix_advance();
+    };
+    // This lane's nibble of K-step ks is nibble 4 (ks & 1) + g of index word ks / 2.  Shifting the
+    // word left by 4 for even g puts that nibble into the high half of byte 2 (ks & 1) + g / 2, so
+    // after masking, one v_bfe_u32 yields nibble * 16: the byte offset of the one-hot table entry.
+    const uint32_t pre_shift = (g & 1) ? 0u : 4u;
+    const uint32_t byte_shift = 8 * (g >> 1);
+    const uint32_t ix_lane = IBUF0 + wave * IWAVE + j * 4;
+    // The index words are read with inline assembly: the compiler cannot tell these reads from the
+    // LDS ranges the copy operations in flight are writing, and would wait for all of them first.
+    auto read_ix = [&](uint32_t (&raw)[TM][IWORDS], uint32_t ibuf) {
+        const uint32_t addr = ix_lane + ibuf * IBYTES;
+        static_for<0, TM * IWORDS>([&](auto ec) {
+            constexpr int t = decltype(ec)::value / IWORDS, i = decltype(ec)::value % IWORDS;
+            lds_read32<(i * 64 + t * 16) * 4>(raw[t][i], addr);
+        });
+    };
+    auto unpack_ix = [&](uint32_t (&iwm)[TM][IWORDS], uint32_t (&raw)[TM][IWORDS]) {
+        static_assert(TM == 4 && (IWORDS == 2 || IWORDS == 4), "operand list of the wait");
+        if constexpr (IWORDS == 2)
+            asm volatile("s_waitcnt lgkmcnt(0)"
+                         : "+v"(raw[0][0]), "+v"(raw[0][1]), "+v"(raw[1][0]), "+v"(raw[1][1]), "+v"(raw[2][0]),
+                           "+v"(raw[2][1]), "+v"(raw[3][0]), "+v"(raw[3][1]));
+        else
+            asm volatile("s_waitcnt lgkmcnt(0)"
+                         : "+v"(raw[0][0]), "+v"(raw[0][1]), "+v"(raw[0][2 % IWORDS]), "+v"(raw[0][3 % IWORDS]),
+                           "+v"(raw[1][0]), "+v"(raw[1][1]), "+v"(raw[1][2 % IWORDS]), "+v"(raw[1][3 % IWORDS]),
+                           "+v"(raw[2][0]), "+v"(raw[2][1]), "+v"(raw[2][2 % IWORDS]), "+v"(raw[2][3 % IWORDS]),
+                           "+v"(raw[3][0]), "+v"(raw[3][1]), "+v"(raw[3][2 % IWORDS]), "+v"(raw[3][3 % IWORDS]));
+#pragma unroll
+        for (int t = 0; t < TM; ++t)
+#pragma unroll
+            for (int i = 0; i < IWORDS; ++i) iwm[t][i] = (raw[t][i] << pre_shift) & 0xF0F0F0F0u;
+    };
+
+    v4i acc[TM][TN];
+#pragma unroll
+    for (int t = 0; t < TM; ++t)
+#pragma unroll
+        for (int c = 0; c < TN; ++c) acc[t][c] = (v4i){0, 0, 0, 0};
+
+    auto epilogue = [&](uint32_t item) -> bool {
+        // j and g pass through an opaque asm so that none of the address arithmetic below is
+        // loop-invariant for the compiler: hoisted out of the slice loop it would occupy dozens of
+        // registers for the whole kernel
+        uint32_t je = j, ge = g;
+        asm volatile("" : "+v"(je), "+v"(ge));
+        const uint32_t colblk = item / n_token_tiles;
+        const uint32_t tile_tok0 = (item % n_token_tiles) * OH_TOK_ITEM;
+        const uint32_t tok0 = tile_tok0 + wave * (TM * 16);
+        const bool vec_store = (M % 4 == 0);
+        const bool full = vec_store && !acc_out && tile_tok0 + OH_TOK_ITEM <= N && (colblk + 1) * WN <= M;
+#pragma unroll
+        for (int c = 0; c < TN; ++c) {
+            const uint32_t f = colblk * WN + c * 16 + 4 * ge;
+            float4 bv = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (ep.bias && f < M) {
+                if (vec_store) {
+                    bv = *reinterpret_cast<const float4*>(ep.bias + f);
+                } else {
+                    bv.x = ep.bias[f];
+                    if (f + 1 < M) bv.y = ep.bias[f + 1];
+                    if (f + 2 < M) bv.z = ep.bias[f + 2];
+                    if (f + 3 < M) bv.w = ep.bias[f + 3];
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < TM; ++t) {
+                const uint32_t tok = tok0 + t * 16 + je;
+                const v4i a = acc[t][c];
+                acc[t][c] = (v4i){0, 0, 0, 0};
+                if (tok >= N || f >= M) continue;
+                float4 o;
+                o.x = dequant(a[0], ep.scale, ep.lut_bias_term, bv.x);
+                o.y = dequant(a[1], ep.scale, ep.lut_bias_term, bv.y);
+                o.z = dequant(a[2], ep.scale, ep.lut_bias_term, bv.z);
+                o.w = dequant(a[3], ep.scale, ep.lut_bias_term, bv.w);
+                if (vec_store) {  // M % 4 == 0 and f % 4 == 0: the whole float4 is in range and aligned
+                    *reinterpret_cast<float4*>(out + (size_t)tok * M + f) = o;
+                    if (acc_out) *reinterpret_cast<v4i*>(acc_out + (size_t)tok * M + f) = a;
+                } else {
+                    const float ov[4] = {o.x, o.y, o.z, o.w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (f + e < M) {
+                            out[(size_t)tok * M + f + e] = ov[e];
+                            if (acc_out) acc_out[(size_t)tok * M + f + e] = a[e];
+                        }
+                    }
+                }
+            }
+        }
+        return full;
+    };
+
+    // ---- prologue: slices 0 .. PD-1, index words 0 .. PD ------------------------------------------
+    locate_lut();
+    locate_ix();
+    static_for<0, PD + 1>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        if (i < total) stage_ix(i);
+    });
+    static_for<0, PD>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        if (i < total) stage_lut(i);
+    });
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();  // also: the one-hot table is complete
+    uint32_t iwm[TM][IWORDS], iw_raw[TM][IWORDS];
+    read_ix(iw_raw, 0);
+    unpack_ix(iwm, iw_raw);
+
+    uint32_t item0 = blockIdx.x;  // the item being consumed
+    const uint32_t a_lane = BUF0 + (g * WN + j) * 16;
+    uint32_t buf = 0, ibuf_next = 1;  // k % NBUF and (k + 1) % NIBUF
+    uint32_t k = 0;                   // position in the flat (item, slice) stream
+    // number of stores a wave issues in the epilogue of a full tile (no tail in tokens or columns,
+    // float4 stores, no accumulator dump): then, and only then, the count is the same for every wave
+    constexpr int EPI_STORES = TM * TN;
+    static_assert((PD - 1) * DMA_OPS + EPI_STORES <= 63, "memory counter range");
+    bool stores_behind = false;       // the previous item's EPI_STORES stores were issued after its last copy operations
+
+    for (uint32_t it = 0; it < my_items; ++it, item0 += gridDim.x) {
+    for (uint32_t s0 = 0; s0 < nslices; ++s0, ++k) {
+        // Loads complete in order, so "at most the (PD-1)*DMA_OPS operations issued during the
+        // previous PD-1 slices are outstanding" means this wave's share of slice k (and of index
+        // words k+1) has landed.  After the barrier everybody's has, and everybody is done with
+        // slice k-1, whose buffer slice k+PD goes into.  The copy operations are issued for every
+        // slice, also past the end of the stream, so the count never changes -- except that the
+        // stores of an item's epilogue sit behind them at the first slice of the next item: when
+        // their number is known they are allowed to stay outstanding (they have had no time to
+        // drain yet), otherwise the wait is simply stricter than necessary.
+        if (k != 0) {
+            if (stores_behind) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((PD - 1) * DMA_OPS + EPI_STORES) : "memory");
+            else asm volatile("s_waitcnt vmcnt(%0)" ::"n"((PD - 1) * DMA_OPS) : "memory");
+            stores_behind = false;
+            __syncthreads();
+        }
+        // This slice's DMA_OPS copy operations (slice k+PD of the LUT, index words k+PD+1) are
+        // issued a few at a time between the K-steps: issued together right after the barrier they
+        // would hold every wave of the CU at the memory pipeline's queue while the matrix core idles.
+        const bool fetch = k + PD < total;            // workgroup-uniform
+        const bool fetch_ix = k + PD + 1 < total;     // workgroup-uniform
+        const uint32_t lbp = buf >= 1 ? buf - 1 : NBUF - 1;               // (k + PD) % NBUF = (k - 1) % NBUF
+        const uint32_t ibp = ibuf_next >= 1 ? ibuf_next - 1 : NIBUF - 1;  // (k + PD + 1) % NIBUF = k % NIBUF
+        const uint32_t abase = buf * SLICE + a_lane;
+
+        v4i a_op[2][TN], b_op[2][TM];
+        // K-step ks covers codebooks 4 ks .. 4 ks + 3 of the slice; this lane's is 4 ks + g.
+        // The operands of K-step ks+1 are requested before the MFMAs of K-step ks are issued.
+        auto issue_reads = [&](auto ksc) {
+            constexpr int ks = decltype(ksc)::value;
+            static_for<0, TN>([&](auto cc) {
+                constexpr int c = decltype(cc)::value;
+                lds_read<(4 * ks * WN + c * 16) * 16>(a_op[ks & 1][c], abase);
+            });
+#pragma unroll
+            for (int t = 0; t < TM; ++t) {
+                const uint32_t entry = __builtin_amdgcn_ubfe(iwm[t][ks / 2], 16 * (ks & 1) + byte_shift, 8);
+                lds_read<0>(b_op[ks & 1][t], entry);
+            }
+        };
+        issue_reads(std::integral_constant<int, 0>{});
+        static_for<0, KSTEPS>([&](auto ksc) {
+            constexpr int ks = decltype(ksc)::value;
+            oh_wait<TN>(a_op[ks & 1], b_op[ks & 1]);
+            if constexpr (ks + 1 < KSTEPS) issue_reads(std::integral_constant<int, ks + 1>{});
+            // the next slice's index words (this wave's own copy, landed before the wait above)
+            if constexpr (ks == KSTEPS - 1) read_ix(iw_raw, ibuf_next);
+            static_for<ks * DMA_OPS / KSTEPS, (ks + 1) * DMA_OPS / KSTEPS>([&](auto oc) {
+                constexpr int o = decltype(oc)::value;
+                if constexpr (o < DMA_PER_WAVE) lut_op(lbp, fetch, std::integral_constant<int, o>{});
+                else ix_op(ibp, fetch_ix, std::integral_constant<int, o - DMA_PER_WAVE>{});
+            });
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int t = 0; t < TM; ++t)
+#pragma unroll
+                for (int c = 0; c < TN; ++c)
+                    acc[t][c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a_op[ks & 1][c], b_op[ks & 1][t], acc[t][c], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        if (fetch) {
+            lut_advance();
+            if (fetch_ix) ix_advance();
+        }
+        unpack_ix(iwm, iw_raw);
+
+        buf = buf + 1 == NBUF ? 0 : buf + 1;
+        ibuf_next = ibuf_next + 1 == NIBUF ? 0 : ibuf_next + 1;
+    }
+    stores_behind = epilogue(item0);
+    }
+}
+
+template <int TN>
+int launch_onehot(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_t* d_acc, uint32_t n,
+                  const Epilogue& ep)
+{
+    constexpr int LDS = oh_lds_bytes(TN);
+    auto kern = gather_onehot_kernel<TN>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        int rc = hip_check(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, LDS),
+                           "hipFuncSetAttribute(gather_onehot)");
+        if (rc) return rc;
+        attr_set = true;
+    }
+    const uint32_t n_token_tiles = (n + OH_TOK_ITEM - 1) / OH_TOK_ITEM;
+    const uint32_t n_items = n_token_tiles * (a.g.M_pad / (16 * TN));
+    uint32_t grid = ctx->prop.multiProcessorCount * 2;  // two workgroups per CU, see plan_geometry
+    if (grid > n_items) grid = n_items;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(OH_THREADS), LDS, ctx->stream, d_idx,
+                       reinterpret_cast<const int8_t*>(a.d_lut), d_out, d_acc, n, a.g.M, a.g.CB_pad,
+                       a.g.idx_row_bytes, n_token_tiles, n_items, ep);
+    return hip_check(ctx, hipGetLastError(), "gather_onehot_kernel launch");
+}
+
 // ---------------------------------------------------------------------------------------------
 // fp32 LUT: out[n][f] = (sum over cb ascending, fp32) lut[cb][idx][f] + bias[f]
 // One lane = one token; a workgroup = 256 tokens x 4*Q columns; slices of GS codebooks in LDS.
@@ -561,6 +958,17 @@ int launch_f32(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, uint3
 //   64    (4, 2)  40 KB                      (4, 8)  40 KB
 //   128   (2, 2)  48 KB                      (2, 8)  48 KB
 //   256   (2, 1)  48 KB                      (2, 4)  48 KB
+// PIMDL_GATHER_ROWS=1 in the environment keeps the byte-adder kernel for every shape (the one-hot
+// kernel gives the same bits; this is for comparing the two).
+bool gather_rows_only()
+{
+    static const bool v = [] {
+        const char* e = getenv("PIMDL_GATHER_ROWS");
+        return e && e[0] == '1';
+    }();
+    return v;
+}
+
 bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::string* why)
 {
     const uint32_t K = d.input_feature_len, v = d.sub_vec_len, C = d.num_centroid, M = d.output_feature_len;
@@ -578,6 +986,40 @@ bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::s
     g->idx_row_bytes = g->CB_pad * g->idx_bits / 8;
     const bool i8 = d.lut_dtype == PIMDL_LUT_I8;
     g->q = ct >= 128 ? 2 : 4;
+    // the one-hot kernel addresses index rows with 32-bit offsets
+    const bool idx_fits = (uint64_t)d.max_n * g->idx_row_bytes <= 0xFFFFFFFFull;
+    g->gather_kind = (i8 && C <= 16 && idx_fits && !gather_rows_only()) ? 1 : 0;
+    if (g->gather_kind == 1) {
+        // One-hot matrix-core kernel: an item is 256 tokens x 16*TN columns, all items cost the
+        // same.  Take the TN that fills the persistent grid (two workgroups per CU) most evenly for
+        // the largest batch this operator will see; among equals the widest (fewest LDS reads).
+        g->C_tile = 16;
+        const uint32_t slots = 2 * (num_cus ? num_cus : 256);
+        const uint32_t tiles = (d.max_n + 255) / 256;
+        double best = -1.0;
+        for (uint32_t tn : {6u, 4u, 3u}) {
+            const uint32_t blocks = (M + 16 * tn - 1) / (16 * tn);
+            const uint64_t items = (uint64_t)tiles * blocks;
+            const uint64_t rounds = (items + slots - 1) / slots;
+            const double eff = (double)items / (double)(rounds * slots) * (double)M / (double)(blocks * 16 * tn);
+            if (eff > best + 1e-9) {
+                best = eff;
+                g->q = tn;
+            }
+        }
+        g->gq = 4;
+        g->cb_per_slice = 16;
+        g->col_block = 16 * g->q;
+        g->gather_threads = 256;
+        g->tokens_per_wg = 256;
+        g->row_pitch = 16;
+        g->gather_lds_bytes = 256 + 3 * (g->cb_per_slice * g->col_block * 16 + 256 * (g->cb_per_slice / 2));
+        g->M_pad = (M + g->col_block - 1) / g->col_block * g->col_block;
+        g->ccs_cb_per_wg = ccs_cb_per_wg(v);
+        g->ccs_row_floats = g->ccs_cb_per_wg * v;
+        g->ccs_lds_bytes = g->ccs_cb_per_wg ? 64 * (g->ccs_row_floats + 4) * 4 : 0;
+        return true;
+    }
     if (i8 && ct >= 16 && ct <= 64) {
         // Column block of 64 or 48 columns: take the one that fills the persistent grid (two
         // workgroups per CU) more evenly for the largest batch this operator will see.  An item is
@@ -627,6 +1069,14 @@ int launch_gather(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, in
         ep.scale = a.h_scale0;
         ep.lut_bias_term = a.desc.bias_mode == PIMDL_BIAS_TIMES_CB ? a.desc.lut_bias * (float)g.CB : a.desc.lut_bias;
         ep.bias = a.d_bias;
+        if (g.gather_kind == 1) {
+            switch (g.q) {
+                case 3: return launch_onehot<3>(ctx, a, d_idx, d_out, d_acc, n, ep);
+                case 4: return launch_onehot<4>(ctx, a, d_idx, d_out, d_acc, n, ep);
+                case 6: return launch_onehot<6>(ctx, a, d_idx, d_out, d_acc, n, ep);
+            }
+            return set_error(ctx, PIMDL_ERR_UNSUPPORTED, "no one-hot gather kernel for %u column groups", g.q);
+        }
         switch (g.C_tile) {
             case 8: return launch_i8<8, 4, 8, 2, 4>(ctx, a, d_idx, d_out, d_acc, n, ep);
             case 16:

@@ -131,6 +131,18 @@ static void retile_lut(const T* lut, T* tiled, const AmmGeom& g, uint32_t row_el
             }
 }
 
+// canonical [CB][C][M] -> [M_pad/col_block][CB_pad][col_block][16], zero padded (C <= 16)
+static void retile_lut_onehot(const int8_t* lut, int8_t* tiled, const AmmGeom& g)
+{
+    const uint32_t wn = g.col_block;
+    for (uint32_t cb = 0; cb < g.CB; ++cb)
+        for (uint32_t c = 0; c < g.C; ++c) {
+            const int8_t* src = lut + ((size_t)cb * g.C + c) * g.M;
+            for (uint32_t f = 0; f < g.M; ++f)
+                tiled[((((size_t)(f / wn) * g.CB_pad + cb) * wn) + f % wn) * 16 + c] = src[f];
+        }
+}
+
 }  // namespace pimdl
 
 using namespace pimdl;
@@ -264,7 +276,8 @@ int pimdl_amm_create(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const float* ce
         delete a;
         return set_error(ctx, PIMDL_ERR_NOMEM, "pimdl_amm_create: host staging of %zu bytes failed", a->lut_bytes);
     }
-    if (i8) retile_lut(reinterpret_cast<const int8_t*>(lut), reinterpret_cast<int8_t*>(tiled.data()), g, row_elems);
+    if (i8 && g.gather_kind == 1) retile_lut_onehot(reinterpret_cast<const int8_t*>(lut), reinterpret_cast<int8_t*>(tiled.data()), g);
+    else if (i8) retile_lut(reinterpret_cast<const int8_t*>(lut), reinterpret_cast<int8_t*>(tiled.data()), g, row_elems);
     else retile_lut(reinterpret_cast<const float*>(lut), reinterpret_cast<float*>(tiled.data()), g, row_elems);
 
     rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&a->d_centroids), ccs_centroid_bytes(g)), "hipMalloc(centroids)");

@@ -14,15 +14,18 @@ namespace pimdl {
 //
 // Index rows   [N][idx_row_bytes] bytes; IDX_BITS = 4 (C <= 16, codebook 2k in the low nibble
 //              of byte k) or 8.  Codebooks are padded to a multiple of 32 with index 0.
-// int8 LUT     tiled [M_pad / col_block][CB_pad][C_tile][col_block] bytes (col_block = 16*Q):
-//              one (column block, codebook range) slice is contiguous, so staging it into LDS
-//              is a flat copy.  Padded codebooks / centroid rows / columns hold zeros.
+// int8 LUT     gather_kind 0: tiled [M_pad / col_block][CB_pad][C_tile][col_block] bytes
+//              (col_block = 16*Q); gather_kind 1: [M_pad / col_block][CB_pad][col_block][16] bytes
+//              (the 16 centroid entries of a column are contiguous).  Either way one (column block,
+//              codebook range) slice is contiguous, so staging it into LDS is a flat copy.  Padded
+//              codebooks / centroid rows / columns hold zeros.
 // fp32 LUT     tiled the same way with col_block floats per row.
 // ---------------------------------------------------------------------------------------------
 struct AmmGeom {
     uint32_t K, v, CB, CB_pad, C, C_tile, M, M_pad;
     uint32_t idx_bits, idx_row_bytes;
     // gather kernel
+    uint32_t gather_kind;   // 0: byte-adder rows kernel, 1: one-hot matrix-core kernel (int8, C <= 16)
     uint32_t q;             // 16-byte chunks per LUT row in LDS
     uint32_t col_block;     // columns per workgroup (int8: 16*q, fp32: 4*q)
     uint32_t row_pitch;     // bytes between LUT rows in LDS (16*q + 16: bank-conflict-free b128 gathers)
@@ -98,6 +101,7 @@ int launch_lut_quant(Ctx* ctx, const float* d_lut, int8_t* d_q, float* d_scales,
 int launch_diag(Ctx* ctx, uint64_t bytes, float* copy_gbps, float* lds_gbps);
 
 uint32_t ccs_cb_per_wg(uint32_t v);  // codebooks one ccs workgroup covers (0: generic kernel)
+bool gather_rows_only();
 bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::string* why);
 
 }  // namespace pimdl
