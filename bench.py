@@ -26,11 +26,12 @@ HBM_PEAK_GBPS = 8000.0                     # MI355X HBM3E
 # WRITE_SIZE by 1.0: the factors a streaming kernel of known size gives for the same counters on
 # this part.  Summary: profiles/bench_ffn_pair_hbm_traffic.txt.  Keyed by (K, M).
 MEASURED_GATHER_TRAFFIC = {
-    (768, 3072): {"fetch_kib": 37581.4, "write_kib": 101973.0},
-    (3072, 768): {"fetch_kib": 39011.9, "write_kib": 24748.0},
+    (768, 3072): {"fetch_kib": 37607.5, "write_kib": 104023.9},
+    (3072, 768): {"fetch_kib": 38545.0, "write_kib": 25934.1},
 }
 FETCH_SCALE, WRITE_SCALE = 2.0, 1.0
 LDS_PEAK_GBPS = 256 * 256 * 2.4            # 256 CUs x 256 B/clk (ds_read_b128) x 2.4 GHz = 157286 GB/s
+MFMA_I8_PEAK_TOPS = 5000.0                 # MI355X dense int8 matrix peak
 
 
 def synth_amm(rng, K, v, C, M, pimdl, ctx):
@@ -179,17 +180,31 @@ def main():
     _, lds_measured = ctx.diag_bandwidth(copy=False, lds=True)
     mt = MEASURED_GATHER_TRAFFIC.get((K, M)) if N == 8192 else None
     traffic = (mt["fetch_kib"] * FETCH_SCALE + mt["write_kib"] * WRITE_SCALE) * 1024.0 if mt else None
+    # The gather for C <= 16 runs as a one-hot int8 matrix product on the MFMA units: per launch it
+    # executes 2 * N * (CB * 16) * M int8 operations to perform the N * CB * M algorithmic adds.
+    one_hot = C <= 16
+    mfma_ops = 2.0 * N * (K // v) * 16 * M
+    mfma_tops = mfma_ops / (dom["gather_ms"] * 1e-3) / 1e12
     roofline = {
-        "kernel": f"gather_i8_kernel ({dom['name']}: K={K} M={M})",
-        "bound": "lds", "achieved": dom["gather_lds_gbps"], "peak": LDS_PEAK_GBPS, "unit": "GB/s",
-        "frac": dom["gather_lds_frac"],
+        "kernel": f"gather_onehot_kernel ({dom['name']}: K={K} M={M})" if one_hot
+                  else f"gather_i8_kernel ({dom['name']}: K={K} M={M})",
+        "bound": "mfma" if one_hot else "lds",
+        "achieved": mfma_tops if one_hot else dom["gather_lds_gbps"],
+        "peak": MFMA_I8_PEAK_TOPS if one_hot else LDS_PEAK_GBPS,
+        "unit": "TOP/s" if one_hot else "GB/s",
+        "frac": (mfma_tops / MFMA_I8_PEAK_TOPS) if one_hot else dom["gather_lds_frac"],
         "traffic": traffic,
         "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this script, scaled x2.0 / x1.0 "
                           "(copy-kernel calibration); recorded constant, not collected in this run",
-        "algorithmic_bytes_per_launch": ab["gather_lds"],
+        "executed_int8_ops_per_launch": mfma_ops,
+        "algorithmic_adds_per_launch": ab["gather_lds"],
         "avg_launch_ms": dom["gather_ms"],
-        "lds_peak_measured_gbps": lds_measured,
-        "frac_of_measured_lds_peak": dom["gather_lds_gbps"] / lds_measured if lds_measured else None,
+        # the same launch against the LDS-gather roofline the metric is worded in: bytes of LUT
+        # entries gathered per second (N*CB*M bytes per launch) over the LDS read peak
+        "lds": {"achieved": dom["gather_lds_gbps"], "peak": LDS_PEAK_GBPS, "unit": "GB/s",
+                "frac": dom["gather_lds_frac"], "algorithmic_bytes_per_launch": ab["gather_lds"],
+                "lds_peak_measured_gbps": lds_measured,
+                "frac_of_measured_lds_peak": dom["gather_lds_gbps"] / lds_measured if lds_measured else None},
         "hbm": {"achieved": dom["gather_hbm_gbps"], "peak": HBM_PEAK_GBPS, "frac": dom["gather_hbm_frac"],
                 "algorithmic_bytes_per_launch": ab["gather_hbm"]},
     }
