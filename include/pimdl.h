@@ -178,6 +178,16 @@ PIMDL_API int pimdl_lutgen(pimdl_ctx* ctx, const float* centroids, const float* 
                            uint32_t output_feature_len, uint32_t lut_dtype, uint32_t scale_group,
                            void* lut_out, float* scales_out);
 
+/* ---- layer normalisation of the transformer layer ---------------------------------------------
+ * Replaces norm() (src/host/transformer_layer.cpp:50-90) and, when `residual` is not NULL, the
+ * residual add that follows it in the layer (:476-486, :601-611):
+ *     out[r][i] = residual[r][i] + ((x[r][i] - mean_r) * (1 / sqrtf(var_r + eps))) * weight[i] + bias[i]
+ * mean and variance accumulated in double and rounded to float, every other operation a separately
+ * rounded fp32 operation, as in the reference (which uses eps = 1e-6).  x, residual, out: [n][d];
+ * weight, bias: [d]; host or device pointers; out may alias residual but not x. */
+PIMDL_API int pimdl_layer_norm(pimdl_ctx* ctx, const float* x, const float* weight, const float* bias,
+                               const float* residual, float* out, uint32_t n, uint32_t d, float eps);
+
 /* ---- introspection ---------------------------------------------------------------------------
  * No reference counterpart: figures a benchmark needs to place a kernel on its roofline. */
 typedef struct pimdl_device_info {

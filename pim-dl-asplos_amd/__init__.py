@@ -27,7 +27,7 @@ EXPORTS = ["pimdl_init", "pimdl_destroy", "pimdl_last_error", "pimdl_set_stream"
            "pimdl_amm_create", "pimdl_amm_destroy", "pimdl_amm_run", "pimdl_amm_run_debug",
            "pimdl_amm_profile", "pimdl_index_calculation", "pimdl_amm_index_calculation", "pimdl_lut_gather",
            "pimdl_amm_run_tiled", "pimdl_lut_gather_tiled", "pimdl_lutgen",
-           "pimdl_get_device_info", "pimdl_amm_get_geometry", "pimdl_diag_bandwidth"]
+           "pimdl_layer_norm", "pimdl_get_device_info", "pimdl_amm_get_geometry", "pimdl_diag_bandwidth"]
 
 
 class PimdlError(RuntimeError):
@@ -119,6 +119,7 @@ def lib():
     L.pimdl_lut_gather_tiled.argtypes = [vp, vp, u32, vp, ctypes.POINTER(Tiling)]
     L.pimdl_lut_gather.argtypes = [vp, vp, u32, vp]
     L.pimdl_lutgen.argtypes = [vp, vp, vp, u32, u32, u32, u32, u32, u32, vp, vp]
+    L.pimdl_layer_norm.argtypes = [vp, vp, vp, vp, vp, vp, u32, u32, ctypes.c_float]
     L.pimdl_get_device_info.argtypes = [vp, ctypes.POINTER(DeviceInfo)]
     L.pimdl_amm_get_geometry.argtypes = [vp, ctypes.POINTER(AmmGeometry)]
     L.pimdl_diag_bandwidth.argtypes = [vp, u64, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float)]
@@ -207,6 +208,26 @@ class Context:
         self._check(lib().pimdl_lutgen(self._h, _ptr(centroids), _ptr(weight), CB, C, v, M, lut_dtype, scale_group,
                                        _ptr(out), _ptr(scales)))
         return out, scales
+
+    def layer_norm(self, x, weight, bias, residual=None, out=None, eps=1e-6):
+        """norm() of the reference's layer (transformer_layer.cpp:50-90), plus the residual add when
+        `residual` is given.  numpy arrays in, numpy array out; or raw addresses (ints) with n, d
+        taken from `x` = (address, n, d) and `out` an address."""
+        if isinstance(x, tuple):
+            addr, n, d = x
+            self._check(lib().pimdl_layer_norm(self._h, _ptr(addr), _ptr(weight), _ptr(bias), _ptr(residual),
+                                               _ptr(out), n, d, ctypes.c_float(eps)))
+            return None
+        x = np.ascontiguousarray(x, np.float32)
+        n, d = x.shape
+        weight = np.ascontiguousarray(weight, np.float32)
+        bias = np.ascontiguousarray(bias, np.float32)
+        if residual is not None:
+            residual = np.ascontiguousarray(residual, np.float32)
+        y = np.empty_like(x)
+        self._check(lib().pimdl_layer_norm(self._h, _ptr(x), _ptr(weight), _ptr(bias), _ptr(residual), _ptr(y), n, d,
+                                           ctypes.c_float(eps)))
+        return y
 
     def amm(self, centroids, lut, scales=None, bias=None, max_n=8192, lut_bias=0.0, bias_mode=BIAS_ONCE,
             scale_group=0):

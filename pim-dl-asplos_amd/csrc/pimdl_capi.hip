@@ -584,6 +584,50 @@ int pimdl_amm_get_geometry(const pimdl_amm* a, pimdl_amm_geometry* out)
     return PIMDL_OK;
 }
 
+int pimdl_layer_norm(pimdl_ctx* ctx, const float* x, const float* weight, const float* bias, const float* residual,
+                     float* out, uint32_t n, uint32_t d, float eps)
+{
+    if (!ctx) return PIMDL_ERR_INVALID;
+    if (!x || !weight || !bias || !out) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_layer_norm: null buffer");
+    if (d == 0) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_layer_norm: zero-sized row");
+    int rc = activate(ctx);
+    if (rc || n == 0) return rc;
+    // every buffer may be a host or a device pointer; host buffers go through temporary device copies
+    const size_t row_bytes = (size_t)d * sizeof(float), mat_bytes = (size_t)n * row_bytes;
+    struct Tmp {
+        void* p = nullptr;
+        ~Tmp() { (void)hipFree(p); }
+    } tx, tw, tb, tr, to;
+    auto to_dev = [&](const float* h, size_t bytes, Tmp& t, const float** dptr) -> int {
+        if (is_device_ptr(h)) {
+            *dptr = h;
+            return PIMDL_OK;
+        }
+        int r = hip_check(ctx, hipMalloc(&t.p, bytes), "hipMalloc(layer_norm staging)");
+        if (!r) r = hip_check(ctx, hipMemcpyAsync(t.p, h, bytes, hipMemcpyHostToDevice, ctx->stream), "H2D layer_norm");
+        *dptr = static_cast<const float*>(t.p);
+        return r;
+    };
+    const float *dx, *dw, *db, *dr = nullptr;
+    if ((rc = to_dev(x, mat_bytes, tx, &dx))) return rc;
+    if ((rc = to_dev(weight, row_bytes, tw, &dw))) return rc;
+    if ((rc = to_dev(bias, row_bytes, tb, &db))) return rc;
+    if (residual && (rc = to_dev(residual, mat_bytes, tr, &dr))) return rc;
+    const bool out_host = !is_device_ptr(out);
+    float* dout = out;
+    if (out_host) {
+        if ((rc = hip_check(ctx, hipMalloc(&to.p, mat_bytes), "hipMalloc(layer_norm staging)"))) return rc;
+        dout = static_cast<float*>(to.p);
+    }
+    if ((rc = launch_layer_norm(ctx, dx, dw, db, dr, dout, n, d, eps))) return rc;
+    if (out_host) {
+        if ((rc = hip_check(ctx, hipMemcpyAsync(out, dout, mat_bytes, hipMemcpyDeviceToHost, ctx->stream), "D2H layer_norm"))) return rc;
+    }
+    if (out_host || tx.p || tw.p || tb.p || tr.p)  // temporaries die at return
+        return hip_check(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+    return PIMDL_OK;
+}
+
 int pimdl_diag_bandwidth(pimdl_ctx* ctx, uint64_t bytes, float* copy_gbps, float* lds_gbps)
 {
     if (!ctx) return PIMDL_ERR_INVALID;

@@ -98,6 +98,8 @@ int launch_lutgen_f32(Ctx* ctx, const float* d_cent, const float* d_w, float* d_
                       uint32_t C, uint32_t v, uint32_t M);
 int launch_lut_quant(Ctx* ctx, const float* d_lut, int8_t* d_q, float* d_scales, uint32_t CB, uint32_t C,
                      uint32_t M, uint32_t scale_group);
+int launch_layer_norm(Ctx* ctx, const float* d_x, const float* d_w, const float* d_b, const float* d_residual,
+                      float* d_out, uint32_t n, uint32_t d, float eps);
 int launch_diag(Ctx* ctx, uint64_t bytes, float* copy_gbps, float* lds_gbps);
 
 uint32_t ccs_cb_per_wg(uint32_t v);  // codebooks one ccs workgroup covers (0: generic kernel)

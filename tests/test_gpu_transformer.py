@@ -1,0 +1,146 @@
+"""The layer/model wrapper on the GPU, checked stage by stage against the CPU oracle.
+
+LUT-AMM is discontinuous (a centroid index can flip on a 1e-7 change of its input), so a whole layer is not
+compared end to end against a CPU layer: each stage is compared against the oracle *given the GPU's own
+input to that stage*.  Bars: every AMM bit-exact; layer normalisation within 1e-5 relative (the two
+double-precision sums run in a different order than the reference's sequential loop); attention and GELU
+(textbook fp32 definitions; the reference's ggml versions are pinned by none of its tests) within 1e-4."""
+import math
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from __graft_entry__ import load_package
+
+pimdl = load_package()
+from pim_dl_asplos_amd import transformer as T  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+HERE = os.path.dirname(os.path.abspath(__file__))
+CFG = os.path.join(HERE, "golden", "transformer_small.yaml")
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    import torch
+    c = pimdl.Context(0)
+    c.set_stream(torch.cuda.current_stream().cuda_stream)
+    yield c
+    c.close()
+
+
+def amm_oracle(w, x):
+    v = w["centroids"].shape[2]
+    CB = w["centroids"].shape[0]
+    idx = oracle.index_calculation(x, w["centroids"], v, threads=8)
+    acc = oracle.gather_i8(idx, w["lut"], threads=8)
+    return oracle.dequant(acc, w["bias"], CB, w["scale"], w.get("lut_bias", 0.0), 1, threads=8)
+
+
+@pytest.mark.parametrize("n,d", [(1, 8), (37, 768), (256, 1024), (5, 100), (3, 4097)])
+def test_layer_norm_matches_the_reference_statement(ctx, n, d):
+    rng = np.random.default_rng(n * 1000 + d)
+    x = (rng.standard_normal((n, d)) * 3 + 0.5).astype(np.float32)
+    w = rng.standard_normal(d).astype(np.float32)
+    b = rng.standard_normal(d).astype(np.float32)
+    r = rng.standard_normal((n, d)).astype(np.float32)
+    want = oracle.layer_norm(x, w, b)
+    got = ctx.layer_norm(x, w, b)
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6)
+    assert (got == want).mean() > 0.99  # in practice the sums round to the same floats
+    got_r = ctx.layer_norm(x, w, b, residual=r)
+    np.testing.assert_allclose(got_r, r + want, rtol=1e-5, atol=1e-6)
+    # a constant row has zero variance: scale = 1/sqrt(eps), output = bias exactly
+    c = np.full((2, d), 1.25, np.float32)
+    assert np.array_equal(ctx.layer_norm(c, w, b), np.broadcast_to(b, (2, d)))
+
+
+def test_layer_stage_by_stage(ctx):
+    import torch
+    p = T.TransformerParams.from_yaml(CFG)
+    layers = T.synth_layers(p, ctx, pimdl, seed=3)
+    rng = np.random.default_rng(9)
+    for name, _ in T.NORMS:  # non-trivial LayerNorm parameters and biases
+        layers[0][name]["weight"] = rng.standard_normal(p.token_dim).astype(np.float32)
+        layers[0][name]["bias"] = rng.standard_normal(p.token_dim).astype(np.float32)
+    for name, _ in T.LINEARS:
+        layers[0][name]["bias"] = rng.standard_normal(layers[0][name]["bias"].shape[0]).astype(np.float32)
+    layer = T.TransformerLayer(ctx, pimdl, layers[0], p)
+    x = rng.standard_normal((p.n, p.token_dim)).astype(np.float32)
+    keep = {}
+    y = layer.forward(torch.from_numpy(x).cuda(), keep)
+    torch.cuda.synchronize()
+    k = {name: t.cpu().numpy() for name, t in keep.items()}
+    w = layers[0]
+    # the six AMMs, each from the GPU's own input: bit-exact
+    for name, src in (("q", x), ("k", x), ("v", x), ("o", k["attn"]), ("ffn1", k["h"]), ("ffn2", k["gelu"])):
+        want = amm_oracle(w[name], np.ascontiguousarray(src))
+        got = k["ffn1" if name == "ffn1" else "ffn2" if name == "ffn2" else name]
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), name
+    # attention: softmax(q k^T / sqrt(head_dim)) v per (batch, head), unmasked
+    B, S, H, hd = p.batch_size, p.seq_len, p.head_num, p.head_dim
+    q, kk, v = (k[n].astype(np.float64).reshape(B, S, H, hd).transpose(0, 2, 1, 3) for n in ("q", "k", "v"))
+    s = q @ kk.transpose(0, 1, 3, 2) / math.sqrt(hd)
+    s = np.exp(s - s.max(-1, keepdims=True))
+    a = (s / s.sum(-1, keepdims=True)) @ v
+    np.testing.assert_allclose(k["attn"], a.transpose(0, 2, 1, 3).reshape(p.n, p.token_dim), rtol=1e-4, atol=1e-4)
+    # residual + LayerNorm, in the reference's placement: h = x + norm(o), y = h + norm(ffn2)
+    np.testing.assert_allclose(k["h"], x + oracle.layer_norm(k["o"], w["attention_norm"]["weight"], w["attention_norm"]["bias"]),
+                               rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(k["out"], k["h"] + oracle.layer_norm(k["ffn2"], w["ffn_norm"]["weight"], w["ffn_norm"]["bias"]),
+                               rtol=1e-5, atol=1e-5)
+    # tanh GELU
+    f = k["ffn1"].astype(np.float64)
+    np.testing.assert_allclose(k["gelu"], 0.5 * f * (1 + np.tanh(math.sqrt(2 / math.pi) * (f + 0.044715 * f ** 3))),
+                               rtol=1e-4, atol=1e-5)
+    assert np.array_equal(y.cpu().numpy(), k["out"])
+    layer.close()
+
+
+def test_fused_qkv_equals_separate_projections(ctx):
+    import torch
+    p = T.TransformerParams.from_yaml(CFG)
+    layers = T.synth_layers(p, ctx, pimdl, seed=4, shared_qkv_centroids=True)
+    w = layers[0]
+    scale = max(w[n]["scale"] for n in "qkv")
+    for n in "qkv":
+        w[n]["scale"] = scale  # one LUT scale for the fused operator
+    x = torch.randn((p.n, p.token_dim), device="cuda", generator=torch.Generator(device="cuda").manual_seed(1))
+    sep, fused = T.TransformerLayer(ctx, pimdl, w, p), T.TransformerLayer(ctx, pimdl, w, p, fused_qkv=True)
+    ks, kf = {}, {}
+    ys, yf = sep.forward(x, ks), fused.forward(x, kf)
+    torch.cuda.synchronize()
+    for n in ("q", "k", "v", "out"):
+        assert torch.equal(ks[n], kf[n]), n
+    assert torch.equal(ys, yf)
+    sep.close()
+    fused.close()
+
+
+def test_model_is_the_chain_of_its_layers_and_reads_the_weight_file(ctx, tmp_path):
+    import torch
+    p = T.TransformerParams.from_yaml(CFG)
+    layers = T.synth_layers(p, ctx, pimdl, seed=5)
+    path = str(tmp_path / "model.npz")
+    T.save_npz(path, layers)
+    model = T.Transformer(ctx, pimdl, T.load_npz(path, p), p)
+    x = torch.randn((p.n, p.token_dim), device="cuda", generator=torch.Generator(device="cuda").manual_seed(2))
+    y = model.forward(x)
+    z = x
+    for w in layers:
+        layer = T.TransformerLayer(ctx, pimdl, w, p)
+        z = layer.forward(z)
+        layer.close()
+    torch.cuda.synchronize()
+    assert torch.equal(y, z)
+    assert torch.isfinite(y).all()
+    model.close()
+
+
+def test_driver_prints_the_reference_wording(capsys):
+    assert T.main([CFG, "--iters", "2"]) == 0
+    out = capsys.readouterr().out
+    assert "weight file is not found, generate weights randomly." in out
+    assert "iteration 1, inference time" in out and "inference end" in out
