@@ -84,3 +84,30 @@ def test_weight_file_that_does_not_match_the_configuration_is_rejected(tmp_path)
     T.save_npz(path, layers)
     with pytest.raises(ValueError):
         T.load_npz(path, p)
+
+
+def test_converter_key_handling_and_shapes():
+    """split_layers / linear_shape follow pim_weight_converter.py:42-55,74-81."""
+    from pim_dl_asplos_amd import convert as CV
+    t = {"bert.embeddings.word_embeddings.weight": np.zeros(3),
+         "bert.encoder.layer.0.attention.self.query.weight": np.zeros(1),
+         "bert.encoder.layer.11.output.dense.centroids.weight": np.zeros(2),
+         "bert.pooler.dense.weight": np.zeros(4),
+         "layer.3.intermediate.dense.bias": np.zeros(5)}
+    layers = CV.split_layers(t)
+    assert sorted(layers) == [0, 3, 11]
+    assert list(layers[0]) == ["0.attention.self.query.weight"]
+    assert list(layers[11]) == ["11.output.dense.centroids.weight"]
+    assert list(layers[3]) == ["3.intermediate.dense.bias"]
+    assert CV.linear_shape("0.attention.self.query", 768) == (768, 768)
+    assert CV.linear_shape("0.attention.output.dense", 768) == (768, 768)
+    assert CV.linear_shape("0.intermediate.dense", 768) == (768, 3072)
+    assert CV.linear_shape("0.output.dense", 768) == (3072, 768)
+    with pytest.raises(ValueError):
+        CV.convert({}, None, None, nsharecodebook=2)
+
+
+def test_shipped_bert_base_configuration_parses():
+    p = T.TransformerParams.from_yaml(os.path.join(HERE, "..", "pim-dl-asplos_amd", "configs", "bert_base_b32_s128.yaml"))
+    assert p.n == 4096 and p.layer_num == 12
+    assert p.shapes["ffn2"].num_codebook == 768 and p.shapes["q"].sub_vec_len == 4
