@@ -104,6 +104,14 @@ PIMDL_API int pimdl_synchronize(pimdl_ctx* ctx);
 PIMDL_API int pimdl_amm_create(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const float* centroids,
                                const void* lut, const float* scales, const float* bias,
                                pimdl_amm** out);
+/* The same with the width of the gather kernel's column tile given by the caller (48, 64 or 96 output
+ * columns; 0 = let the library choose by load balance, which is what pimdl_amm_create does).  This is the
+ * knob a measured tile search turns -- the counterpart of the tile parameters the reference's auto-tuner
+ * writes into its YAML (inference-engine/src/tuner/auto_tuner.cpp:552-603), found by timing instead of by a latency model.
+ * PIMDL_ERR_INVALID if the operator's kernel has no variant of that width. */
+PIMDL_API int pimdl_amm_create_tuned(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const float* centroids,
+                                     const void* lut, const float* scales, const float* bias,
+                                     uint32_t col_block, pimdl_amm** out);
 PIMDL_API int pimdl_amm_destroy(pimdl_amm* amm);
 
 /* The AMM itself.  Replaces amm_host (src/host/amm_host.h:8-10, amm_host.cpp:10-30) =

@@ -19,12 +19,13 @@ CSRC = os.path.join(_HERE, "csrc")
 LUT_I8, LUT_F32 = 0, 1
 BIAS_ONCE, BIAS_TIMES_CB = 0, 1
 
+ERR_INVALID, ERR_UNSUPPORTED, ERR_HIP = -1, -2, -3
 STATUS = {0: "PIMDL_OK", -1: "PIMDL_ERR_INVALID", -2: "PIMDL_ERR_UNSUPPORTED", -3: "PIMDL_ERR_HIP",
           -4: "PIMDL_ERR_NOMEM", -5: "PIMDL_ERR_NO_DEVICE"}
 
 # every symbol include/pimdl.h declares
 EXPORTS = ["pimdl_init", "pimdl_destroy", "pimdl_last_error", "pimdl_set_stream", "pimdl_synchronize",
-           "pimdl_amm_create", "pimdl_amm_destroy", "pimdl_amm_run", "pimdl_amm_run_debug",
+           "pimdl_amm_create", "pimdl_amm_create_tuned", "pimdl_amm_destroy", "pimdl_amm_run", "pimdl_amm_run_debug",
            "pimdl_amm_profile", "pimdl_index_calculation", "pimdl_amm_index_calculation", "pimdl_lut_gather",
            "pimdl_amm_run_tiled", "pimdl_lut_gather_tiled", "pimdl_lutgen",
            "pimdl_layer_norm", "pimdl_get_device_info", "pimdl_amm_get_geometry", "pimdl_diag_bandwidth"]
@@ -109,6 +110,7 @@ def lib():
     L.pimdl_set_stream.argtypes = [vp, vp]
     L.pimdl_synchronize.argtypes = [vp]
     L.pimdl_amm_create.argtypes = [vp, ctypes.POINTER(AmmDesc), vp, vp, vp, vp, ctypes.POINTER(vp)]
+    L.pimdl_amm_create_tuned.argtypes = [vp, ctypes.POINTER(AmmDesc), vp, vp, vp, vp, u32, ctypes.POINTER(vp)]
     L.pimdl_amm_destroy.argtypes = [vp]
     L.pimdl_amm_run.argtypes = [vp, vp, u32, vp]
     L.pimdl_amm_run_debug.argtypes = [vp, vp, u32, vp, vp, vp]
@@ -230,14 +232,15 @@ class Context:
         return y
 
     def amm(self, centroids, lut, scales=None, bias=None, max_n=8192, lut_bias=0.0, bias_mode=BIAS_ONCE,
-            scale_group=0):
-        return Amm(self, centroids, lut, scales, bias, max_n, lut_bias, bias_mode, scale_group)
+            scale_group=0, col_block=0):
+        """col_block: width of the gather kernel's column tile (0 = chosen by the library)."""
+        return Amm(self, centroids, lut, scales, bias, max_n, lut_bias, bias_mode, scale_group, col_block)
 
 
 class Amm:
     """One LUT-AMM operator resident in HBM."""
 
-    def __init__(self, ctx, centroids, lut, scales, bias, max_n, lut_bias, bias_mode, scale_group):
+    def __init__(self, ctx, centroids, lut, scales, bias, max_n, lut_bias, bias_mode, scale_group, col_block=0):
         centroids = np.ascontiguousarray(centroids, np.float32)
         CB, C, v = centroids.shape
         lut = np.ascontiguousarray(lut)
@@ -252,8 +255,8 @@ class Amm:
             bias = np.ascontiguousarray(bias, np.float32)
             assert bias.shape == (M,)
         self._h = ctypes.c_void_p()
-        ctx._check(lib().pimdl_amm_create(ctx._h, ctypes.byref(desc), _ptr(centroids), _ptr(lut), _ptr(scales),
-                                          _ptr(bias), ctypes.byref(self._h)))
+        ctx._check(lib().pimdl_amm_create_tuned(ctx._h, ctypes.byref(desc), _ptr(centroids), _ptr(lut), _ptr(scales),
+                                                _ptr(bias), col_block, ctypes.byref(self._h)))
 
     def close(self):
         if self._h and self.ctx._h:

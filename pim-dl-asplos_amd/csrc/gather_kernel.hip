@@ -969,7 +969,7 @@ bool gather_rows_only()
     return v;
 }
 
-bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::string* why)
+bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::string* why, uint32_t col_block_hint)
 {
     const uint32_t K = d.input_feature_len, v = d.sub_vec_len, C = d.num_centroid, M = d.output_feature_len;
     if (!K || !v || !C || !M || !d.max_n) { *why = "zero-sized dimension"; return false; }
@@ -997,7 +997,12 @@ bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::s
         const uint32_t slots = 2 * (num_cus ? num_cus : 256);
         const uint32_t tiles = (d.max_n + 255) / 256;
         double best = -1.0;
+        if (col_block_hint && col_block_hint != 96 && col_block_hint != 64 && col_block_hint != 48) {
+            *why = "column tile hint must be 48, 64 or 96 for this operator";
+            return false;
+        }
         for (uint32_t tn : {6u, 4u, 3u}) {
+            if (col_block_hint && col_block_hint != 16 * tn) continue;
             const uint32_t blocks = (M + 16 * tn - 1) / (16 * tn);
             const uint64_t items = (uint64_t)tiles * blocks;
             const uint64_t rounds = (items + slots - 1) / slots;
@@ -1027,7 +1032,12 @@ bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::s
         const uint32_t slots = 2 * (num_cus ? num_cus : 256);
         const uint32_t tiles = (d.max_n + 255) / 256;
         double best = -1.0;
+        if (col_block_hint && col_block_hint != 64 && col_block_hint != 48) {
+            *why = "column tile hint must be 48 or 64 for this operator";
+            return false;
+        }
         for (uint32_t q : {4u, 3u}) {
+            if (col_block_hint && col_block_hint != 16 * q) continue;
             const uint32_t blocks = (M + 16 * q - 1) / (16 * q);
             const uint64_t items = (uint64_t)tiles * blocks;
             const uint64_t rounds = (items + slots - 1) / slots;

@@ -238,6 +238,12 @@ int pimdl_synchronize(pimdl_ctx* ctx)
 int pimdl_amm_create(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const float* centroids, const void* lut,
                      const float* scales, const float* bias, pimdl_amm** out)
 {
+    return pimdl_amm_create_tuned(ctx, desc, centroids, lut, scales, bias, 0, out);
+}
+
+int pimdl_amm_create_tuned(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const float* centroids, const void* lut,
+                           const float* scales, const float* bias, uint32_t col_block, pimdl_amm** out)
+{
     if (!ctx) return PIMDL_ERR_INVALID;
     if (!desc || !centroids || !lut || !out) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_create: null argument");
     *out = nullptr;
@@ -246,7 +252,7 @@ int pimdl_amm_create(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const float* ce
     AmmGeom g;
     memset(&g, 0, sizeof(g));
     std::string why;
-    if (!plan_geometry(*desc, ctx->prop.multiProcessorCount, &g, &why)) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_create: %s", why.c_str());
+    if (!plan_geometry(*desc, ctx->prop.multiProcessorCount, &g, &why, col_block)) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_create: %s", why.c_str());
     const bool i8 = desc->lut_dtype == PIMDL_LUT_I8;
     if (i8 && !scales) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_create: int8 LUT needs scales");
     if (i8 && desc->scale_group != 0)

@@ -104,6 +104,9 @@ int launch_diag(Ctx* ctx, uint64_t bytes, float* copy_gbps, float* lds_gbps);
 
 uint32_t ccs_cb_per_wg(uint32_t v);  // codebooks one ccs workgroup covers (0: generic kernel)
 bool gather_rows_only();
-bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::string* why);
+// col_block_hint: 0 = choose the column tile by load balance, else the width to use (an error if this
+// operator's kernel has no such variant)
+bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::string* why,
+                   uint32_t col_block_hint = 0);
 
 }  // namespace pimdl

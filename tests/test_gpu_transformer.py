@@ -144,3 +144,35 @@ def test_driver_prints_the_reference_wording(capsys):
     out = capsys.readouterr().out
     assert "weight file is not found, generate weights randomly." in out
     assert "iteration 1, inference time" in out and "inference end" in out
+
+
+def test_column_tile_hint_and_measured_tile_search(ctx, tmp_path):
+    """Every column-tile width gives the same bits; an unavailable width is rejected; the tuner picks one
+    of the widths it measured and caches it."""
+    from pim_dl_asplos_amd import autotune as AT
+    rng = np.random.default_rng(2)
+    N, K, v, C, M = 300, 64, 4, 16, 200
+    x = rng.standard_normal((N, K)).astype(np.float32)
+    cent = rng.standard_normal((K // v, C, v)).astype(np.float32)
+    lut = rng.integers(-128, 128, (K // v, C, M)).astype(np.int8)
+    outs = []
+    for cb in (0, 48, 64, 96):
+        amm = ctx.amm(cent, lut, np.float32(0.02), None, max_n=N, col_block=cb)
+        assert cb == 0 or amm.geometry()["col_block"] == cb
+        outs.append(amm.run(x))
+        amm.close()
+    for o in outs[1:]:
+        assert np.array_equal(o.view(np.uint32), outs[0].view(np.uint32))
+    with pytest.raises(pimdl.PimdlError) as e:
+        ctx.amm(cent, lut, np.float32(0.02), None, max_n=N, col_block=80)
+    assert e.value.code == pimdl.ERR_INVALID
+    best, results = AT.tune(ctx, pimdl, 512, 128, 4, 16, 384, iters=3)
+    assert best in (48, 64, 96) and best in results and results[best]["gather_ms"] > 0
+    cache = AT.TileCache(str(tmp_path / "tiles.json"))
+    key = AT.shape_key("dev", 512, 128, 4, 16, 384, "int8")
+    cache.put(key, best)
+    assert AT.TileCache(str(tmp_path / "tiles.json")).get(key) == best
+    AT.write_yaml(str(tmp_path / "t.yaml"), 512, 128, 4, 16, 384, best, results[best])
+    import yaml
+    doc = yaml.safe_load(open(str(tmp_path / "t.yaml")))
+    assert doc["amm_shape_params"]["num_codebook"] == 32 and doc["kernel_params"]["col_block"] == best
