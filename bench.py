@@ -55,6 +55,27 @@ def algorithmic_bytes(N, K, v, C, M, e=1):
     }
 
 
+def model_forward(pimdl, ctx, iters=5):
+    """The full 12-layer LUT-BERT-base encoder forward (every linear a LUT-AMM, v=4, C=16, int8 LUTs;
+    N = 32 x 128 = 4096 tokens, random-init weights), timed end to end on the GPU: a secondary figure
+    next to the headline metric."""
+    import torch
+    from pim_dl_asplos_amd import transformer as T
+    p = T.TransformerParams.bert_base(batch_size=32, seq_len=128, layer_num=12)
+    model = T.Transformer(ctx, pimdl, T.synth_layers(p, ctx, pimdl, seed=1), p)
+    x = torch.randn((p.n, p.token_dim), device="cuda", dtype=torch.float32)
+    model.forward(x)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        model.forward(x)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / iters
+    model.close()
+    return {"layers": 12, "tokens": p.n, "ms_per_forward": ms, "tokens_per_s": p.n / (ms * 1e-3),
+            "note": "LUT-AMM linears + pimdl_layer_norm on libpimdl, attention and tanh-GELU in PyTorch-ROCm fp32"}
+
+
 def cpu_baseline(shapes, N, budget_s=12.0):
     """The oracle's restatement of the reference's amm_cpu (test_amm.cpp:126-183), timed on this
     host's cores on a bounded token sample of the same two AMMs."""
@@ -97,6 +118,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--tokens", type=int, default=8192)
+    ap.add_argument("--no-model", action="store_true", help="skip the 12-layer model forward timing")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -226,6 +248,8 @@ def main():
         "per_amm": per_amm,
         "roofline": roofline,
     }
+    if not args.no_model:
+        result["bert_base_forward"] = model_forward(pimdl, ctx)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(shapes, N)
     for a in amms:
