@@ -66,8 +66,12 @@ typedef struct pimdl_amm_desc {
     uint32_t output_feature_len;/* M */
     uint32_t lut_dtype;         /* pimdl_lut_dtype */
     uint32_t scale_group;       /* int8 only. 0: one scale for the tensor (the reference,
-                                   LUTParams.scale).  g > 0 (extension): one scale per g
-                                   consecutive codebooks, int32 inside a group, fp32 across. */
+                                   LUTParams.scale).  g > 0 (extension, no counterpart in the
+                                   reference): one scale per g consecutive codebooks; the sum
+                                   inside a group is exact, then out = (sum over groups
+                                   ascending, fp32, from 0) (float)acc_g * scale[g] + bias[f].
+                                   Needs lut_bias == 0; runs on the fp32-table gather kernel
+                                   (the table is resident as fp32 integers, 4 bytes/entry). */
     uint32_t bias_mode;         /* pimdl_bias_mode */
     float lut_bias;             /* LUTParams.bias */
 } pimdl_amm_desc;

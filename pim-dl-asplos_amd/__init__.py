@@ -251,6 +251,8 @@ class Amm:
         desc = AmmDesc(max_n, CB * v, v, C, M, self.lut_dtype, scale_group, bias_mode, lut_bias)
         if scales is not None:
             scales = np.ascontiguousarray(np.atleast_1d(scales), np.float32)
+            want = (CB + scale_group - 1) // scale_group if (scale_group and self.lut_dtype == LUT_I8) else 1
+            assert scales.size == want, f"{want} scale(s) expected, got {scales.size}"
         if bias is not None:
             bias = np.ascontiguousarray(bias, np.float32)
             assert bias.shape == (M,)

@@ -794,16 +794,24 @@ int launch_onehot(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, in
 // ---------------------------------------------------------------------------------------------
 // fp32 LUT: out[n][f] = (sum over cb ascending, fp32) lut[cb][idx][f] + bias[f]
 // One lane = one token; a workgroup = 256 tokens x 4*Q columns; slices of GS codebooks in LDS.
+//
+// GROUPED (int8 table with one scale per `group` consecutive codebooks; not in the reference): the
+// table holds the int8 entries converted to fp32, so the sum inside a group is an exact integer
+// (|sum| <= 128 * group < 2^24 is checked at creation); at the end of each group
+//     tot = tot + (float)acc_g * scale[g]      (two separately rounded operations, groups ascending)
+// and out = tot + bias[f].
 // ---------------------------------------------------------------------------------------------
 constexpr int GF_THREADS = 256;
 
-template <int C_T, int Q, int GS, int IDX_BITS>
+template <int C_T, int Q, int GS, int IDX_BITS, bool GROUPED>
 __global__ __launch_bounds__(GF_THREADS) void gather_f32_kernel(const uint8_t* __restrict__ idx,
                                                                const float* __restrict__ lut,
                                                                float* __restrict__ out, uint32_t N,
                                                                uint32_t M, uint32_t CB_pad,
                                                                uint32_t idx_row_bytes,
-                                                               const float* __restrict__ bias)
+                                                               const float* __restrict__ bias,
+                                                               const float* __restrict__ scales,
+                                                               uint32_t CB, uint32_t group)
 {
     constexpr int FB = 4 * Q;             // columns per row
     constexpr int PITCH = 16 * Q + 16;    // bytes
@@ -826,6 +834,10 @@ __global__ __launch_bounds__(GF_THREADS) void gather_f32_kernel(const uint8_t* _
     float acc[FB];
 #pragma unroll
     for (int i = 0; i < FB; ++i) acc[i] = 0.0f;
+    float tot[GROUPED ? FB : 1];
+#pragma unroll
+    for (int i = 0; i < (GROUPED ? FB : 1); ++i) tot[i] = 0.0f;
+    uint32_t cb = 0, in_group = 0, gi = 0;  // workgroup-uniform position in the codebook sequence
 
     uint4 stage[UPT];
     uint32_t idx_cur[IDX_WORDS], idx_nxt[IDX_WORDS];
@@ -880,6 +892,20 @@ __global__ __launch_bounds__(GF_THREADS) void gather_f32_kernel(const uint8_t* _
                     acc[4 * c + 2] = __fadd_rn(acc[4 * c + 2], vv.z);
                     acc[4 * c + 3] = __fadd_rn(acc[4 * c + 3], vv.w);
                 }
+                if constexpr (GROUPED) {
+                    // codebooks past CB are padding (zero rows) and belong to no group
+                    if (cb < CB && (++in_group == group || cb + 1 == CB)) {
+                        const float sc = scales[gi];
+#pragma unroll
+                        for (int i = 0; i < FB; ++i) {
+                            tot[i] = __fadd_rn(tot[i], __fmul_rn(acc[i], sc));
+                            acc[i] = 0.0f;
+                        }
+                        ++gi;
+                        in_group = 0;
+                    }
+                    ++cb;
+                }
             }
         }
         PIMDL_COMMIT_SLICE((s + 1) & 1)
@@ -894,7 +920,7 @@ __global__ __launch_bounds__(GF_THREADS) void gather_f32_kernel(const uint8_t* _
 #pragma unroll
         for (int i = 0; i < FB; ++i) {
             const uint32_t f = colblk * FB + i;
-            if (f < M) out[(size_t)tok * M + f] = __fadd_rn(acc[i], bias ? bias[f] : 0.0f);
+            if (f < M) out[(size_t)tok * M + f] = __fadd_rn(GROUPED ? tot[i] : acc[i], bias ? bias[f] : 0.0f);
         }
     }
 }
@@ -927,11 +953,11 @@ int launch_i8(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_
     return hip_check(ctx, hipGetLastError(), "gather_i8_kernel launch");
 }
 
-template <int C_T, int Q, int GS, int IDX_BITS>
-int launch_f32(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, uint32_t n)
+template <int C_T, int Q, int GS, int IDX_BITS, bool GROUPED>
+int launch_f32_impl(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, uint32_t n)
 {
     constexpr int LDS = 2 * GS * C_T * (16 * Q + 16);
-    auto kern = gather_f32_kernel<C_T, Q, GS, IDX_BITS>;
+    auto kern = gather_f32_kernel<C_T, Q, GS, IDX_BITS, GROUPED>;
     static bool attr_set = false;
     if (!attr_set) {
         int rc = hip_check(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -943,8 +969,15 @@ int launch_f32(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, uint3
     dim3 grid((n + GF_THREADS - 1) / GF_THREADS, a.g.M_pad / (4 * Q));
     hipLaunchKernelGGL(kern, grid, dim3(GF_THREADS), LDS, ctx->stream, d_idx,
                        reinterpret_cast<const float*>(a.d_lut), d_out, n, a.g.M, a.g.CB_pad, a.g.idx_row_bytes,
-                       a.d_bias);
+                       a.d_bias, a.d_scales, a.g.CB, a.desc.scale_group);
     return hip_check(ctx, hipGetLastError(), "gather_f32_kernel launch");
+}
+
+template <int C_T, int Q, int GS, int IDX_BITS>
+int launch_f32(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, uint32_t n)
+{
+    return a.grouped ? launch_f32_impl<C_T, Q, GS, IDX_BITS, true>(ctx, a, d_idx, d_out, n)
+                     : launch_f32_impl<C_T, Q, GS, IDX_BITS, false>(ctx, a, d_idx, d_out, n);
 }
 
 }  // namespace
@@ -1074,7 +1107,7 @@ int launch_gather(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, in
 {
     if (n == 0) return PIMDL_OK;
     const AmmGeom& g = a.g;
-    if (a.desc.lut_dtype == PIMDL_LUT_I8) {
+    if (a.desc.lut_dtype == PIMDL_LUT_I8 && !a.grouped) {
         Epilogue ep;
         ep.scale = a.h_scale0;
         ep.lut_bias_term = a.desc.bias_mode == PIMDL_BIAS_TIMES_CB ? a.desc.lut_bias * (float)g.CB : a.desc.lut_bias;

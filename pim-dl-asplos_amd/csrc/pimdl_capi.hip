@@ -249,16 +249,22 @@ int pimdl_amm_create_tuned(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const flo
     *out = nullptr;
     int rc = activate(ctx);
     if (rc) return rc;
+    const bool i8_in = desc->lut_dtype == PIMDL_LUT_I8;
+    // One scale per group of codebooks: the table is kept as fp32 integers and gathered by the
+    // fp32 kernel, which applies scale[g] at the end of each group.
+    const bool grouped = i8_in && desc->scale_group != 0;
+    pimdl_amm_desc plan = *desc;
+    if (grouped) plan.lut_dtype = PIMDL_LUT_F32;
     AmmGeom g;
     memset(&g, 0, sizeof(g));
     std::string why;
-    if (!plan_geometry(*desc, ctx->prop.multiProcessorCount, &g, &why, col_block)) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_create: %s", why.c_str());
-    const bool i8 = desc->lut_dtype == PIMDL_LUT_I8;
-    if (i8 && !scales) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_create: int8 LUT needs scales");
-    if (i8 && desc->scale_group != 0)
-        return set_error(ctx, PIMDL_ERR_UNSUPPORTED,
-                         "pimdl_amm_create: scale_group=%u: only the per-tensor scale (0) is implemented",
-                         desc->scale_group);
+    if (!plan_geometry(plan, ctx->prop.multiProcessorCount, &g, &why, col_block)) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_create: %s", why.c_str());
+    if (i8_in && !scales) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_create: int8 LUT needs scales");
+    if (grouped && desc->lut_bias != 0.0f)
+        return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_create: scale_group > 0 has no zero point: lut_bias must be 0");
+    if (grouped && desc->scale_group > (1u << 16))
+        return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_create: scale_group=%u: a group's sum must stay below 2^24", desc->scale_group);
+    const bool i8 = i8_in && !grouped;  // resident as int8
 
     pimdl_amm* a = new pimdl_amm();
     a->ctx = ctx;
@@ -268,7 +274,8 @@ int pimdl_amm_create_tuned(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const flo
     a->d_lut = nullptr;
     a->d_scales = nullptr;
     a->d_bias = nullptr;
-    a->nscales = i8 ? 1 : 0;
+    a->grouped = grouped;
+    a->nscales = grouped ? (g.CB + desc->scale_group - 1) / desc->scale_group : i8 ? 1 : 0;
     a->h_scale0 = i8 ? scales[0] : 1.0f;
 
     const size_t cent_bytes = (size_t)g.CB * g.C * g.v * sizeof(float);
@@ -284,12 +291,22 @@ int pimdl_amm_create_tuned(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const flo
     }
     if (i8 && g.gather_kind == 1) retile_lut_onehot(reinterpret_cast<const int8_t*>(lut), reinterpret_cast<int8_t*>(tiled.data()), g);
     else if (i8) retile_lut(reinterpret_cast<const int8_t*>(lut), reinterpret_cast<int8_t*>(tiled.data()), g, row_elems);
-    else retile_lut(reinterpret_cast<const float*>(lut), reinterpret_cast<float*>(tiled.data()), g, row_elems);
+    else if (grouped) {
+        std::vector<float> wide;
+        try {
+            const int8_t* q = reinterpret_cast<const int8_t*>(lut);
+            wide.assign(q, q + (size_t)g.CB * g.C * g.M);  // int8 -> float, exact
+        } catch (...) {
+            delete a;
+            return set_error(ctx, PIMDL_ERR_NOMEM, "pimdl_amm_create: host staging of the widened table failed");
+        }
+        retile_lut(wide.data(), reinterpret_cast<float*>(tiled.data()), g, row_elems);
+    } else retile_lut(reinterpret_cast<const float*>(lut), reinterpret_cast<float*>(tiled.data()), g, row_elems);
 
     rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&a->d_centroids), ccs_centroid_bytes(g)), "hipMalloc(centroids)");
     if (!rc) rc = hip_check(ctx, hipMalloc(&a->d_lut, a->lut_bytes), "hipMalloc(lut)");
     if (!rc) rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&a->d_bias), (size_t)g.M * sizeof(float)), "hipMalloc(bias)");
-    if (!rc && i8) rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&a->d_scales), sizeof(float) * a->nscales), "hipMalloc(scales)");
+    if (!rc && a->nscales) rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&a->d_scales), sizeof(float) * a->nscales), "hipMalloc(scales)");
     if (!rc) rc = hip_check(ctx, hipMemcpy(a->d_centroids, centroids, cent_bytes, hipMemcpyHostToDevice), "H2D centroids");
     if (!rc) rc = launch_ccs_prep(ctx, g, a->d_centroids);
     if (!rc) rc = hip_check(ctx, hipMemcpy(a->d_lut, tiled.data(), a->lut_bytes, hipMemcpyHostToDevice), "H2D lut");
@@ -297,7 +314,7 @@ int pimdl_amm_create_tuned(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const flo
         if (bias) rc = hip_check(ctx, hipMemcpy(a->d_bias, bias, (size_t)g.M * sizeof(float), hipMemcpyHostToDevice), "H2D bias");
         else rc = hip_check(ctx, hipMemset(a->d_bias, 0, (size_t)g.M * sizeof(float)), "memset bias");
     }
-    if (!rc && i8) rc = hip_check(ctx, hipMemcpy(a->d_scales, scales, sizeof(float) * a->nscales, hipMemcpyHostToDevice), "H2D scales");
+    if (!rc && a->nscales) rc = hip_check(ctx, hipMemcpy(a->d_scales, scales, sizeof(float) * a->nscales, hipMemcpyHostToDevice), "H2D scales");
     if (rc) {
         pimdl_amm_destroy(a);
         return rc;
@@ -341,8 +358,8 @@ int pimdl_amm_run_debug(pimdl_amm* a, const float* in, uint32_t n, float* out, u
     if (rc || n == 0) return rc;
     Ctx* ctx = a->ctx;
     const AmmGeom& g = a->g;
-    if (acc_out && a->desc.lut_dtype != PIMDL_LUT_I8)
-        return set_error(ctx, PIMDL_ERR_INVALID, "acc_out is only defined for int8 LUTs");
+    if (acc_out && (a->desc.lut_dtype != PIMDL_LUT_I8 || a->grouped))
+        return set_error(ctx, PIMDL_ERR_INVALID, "acc_out is only defined for int8 LUTs with one scale (scale_group 0)");
     const float* d_in;
     float* d_out;
     bool out_host;

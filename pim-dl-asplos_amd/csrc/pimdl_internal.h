@@ -49,6 +49,7 @@ struct Amm {
     uint32_t nscales;
     float* d_bias;       // [M]
     float h_scale0;
+    bool grouped;        // int8 LUT with scale_group > 0: resident as fp32 integers, fp32 gather kernel
 };
 
 struct Ctx {

@@ -167,6 +167,53 @@ def test_fp32_lut_path(ctx, C, v):
     amm.close()
 
 
+@pytest.mark.parametrize("group,C,v,CB,M", [(1, 16, 4, 48, 100), (3, 16, 4, 48, 100), (5, 16, 2, 48, 64),
+                                            (16, 16, 4, 192, 96), (64, 8, 8, 48, 33), (7, 32, 4, 40, 100),
+                                            (4, 64, 4, 20, 72), (2, 256, 2, 6, 40)])
+def test_scale_per_codebook_group(ctx, group, C, v, CB, M):
+    """int8 LUT with one scale per `group` codebooks (an extension the reference does not have, so the
+    only pin is the oracle's definition: int32 inside a group, then fp32 `tot += (float)acc_g * scale[g]`
+    over groups ascending, then + bias).  Bit-exact against it, including ragged last groups, a group
+    larger than CB, 4- and 8-bit index rows; group 1 is BASELINE's per-codebook scale."""
+    N, K = 300, CB * v
+    x, cent, lut, bias = make_case(500 + group + C, N, K, v, C, M)
+    ng = (CB + group - 1) // group
+    scales = np.random.default_rng(group).uniform(1e-3, 0.1, ng).astype(np.float32)
+    amm = ctx.amm(cent, lut, scales, bias, max_n=N, scale_group=group)
+    out = amm.run(x)
+    want_idx = oracle.index_calculation(x, cent, v, threads=THREADS)
+    want = oracle.gather_i8_grouped(want_idx, lut, scales, bias, group, threads=THREADS)
+    assert np.array_equal(out.view(np.uint32), want.view(np.uint32)), \
+        f"{(out.view(np.uint32) != want.view(np.uint32)).sum()} of {out.size} outputs differ"
+    amm.close()
+
+
+def test_scale_groups_from_lutgen(ctx):
+    """lutgen with per-group quantisation -> operator with the same grouping: closer to the fp32 product
+    than the per-tensor quantisation of the same table, and equal to the oracle on the generated table."""
+    rng = np.random.default_rng(77)
+    CB, C, v, M, N = 64, 16, 4, 128, 256
+    cent = rng.standard_normal((CB, C, v)).astype(np.float32)
+    cent[::4] *= 8.0                                     # codebooks of very different magnitude
+    W = (rng.standard_normal((CB * v, M)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((N, CB * v)).astype(np.float32)
+    lut_f, _ = ctx.lutgen(cent, W, lut_dtype=pimdl.LUT_F32)
+    lut_t, s_t = ctx.lutgen(cent, W)
+    lut_g, s_g = ctx.lutgen(cent, W, scale_group=1)
+    assert s_g.shape == (CB,)
+    idx = oracle.index_calculation(x, cent, v, threads=THREADS)
+    exact = oracle.gather_f32(idx, lut_f, np.zeros(M, np.float32), threads=THREADS)
+    a_t = ctx.amm(cent, lut_t, s_t, None, max_n=N)
+    a_g = ctx.amm(cent, lut_g, s_g, None, max_n=N, scale_group=1)
+    out_t, out_g = a_t.run(x), a_g.run(x)
+    want_g = oracle.gather_i8_grouped(idx, lut_g, s_g, np.zeros(M, np.float32), 1, threads=THREADS)
+    assert np.array_equal(out_g.view(np.uint32), want_g.view(np.uint32))
+    err_t, err_g = np.abs(out_t - exact).mean(), np.abs(out_g - exact).mean()
+    assert err_g < 0.7 * err_t, (err_g, err_t)
+    a_t.close()
+    a_g.close()
+
+
 def test_device_pointers_and_partial_batches(ctx):
     """Inputs already resident in HBM (torch tensors), n smaller than max_n, output rows past n untouched."""
     import torch
@@ -196,9 +243,14 @@ def test_error_paths(ctx):
     with pytest.raises(pimdl.PimdlError) as e:
         ctx.amm(cent, lut, None, None)           # int8 LUT without scales
     assert e.value.code == -1
-    with pytest.raises(pimdl.PimdlError) as e:
-        ctx.amm(cent, lut, np.float32(1), None, scale_group=3)
-    assert e.value.code == -2
+    with pytest.raises(pimdl.PimdlError) as e:           # grouped scales have no zero point
+        ctx.amm(cent, lut, np.ones(2, np.float32), None, scale_group=3, lut_bias=0.5)
+    assert e.value.code == -1
+    amm = ctx.amm(cent, lut, np.ones(2, np.float32), None, scale_group=3, max_n=8)
+    with pytest.raises(pimdl.PimdlError) as e:           # no single int32 accumulator to return
+        amm.run_debug(np.zeros((4, 16), np.float32))
+    assert e.value.code == -1
+    amm.close()
     amm = ctx.amm(cent, lut, np.float32(1), None, max_n=8)
     with pytest.raises(pimdl.PimdlError) as e:
         amm.run(np.zeros((9, 16), np.float32))   # n > max_n
