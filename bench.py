@@ -55,7 +55,7 @@ def algorithmic_bytes(N, K, v, C, M, e=1):
     }
 
 
-def model_forward(pimdl, ctx, iters=5):
+def model_forward(pimdl, ctx, iters=10):
     """The full 12-layer LUT-BERT-base encoder forward (every linear a LUT-AMM, v=4, C=16, int8 LUTs;
     N = 32 x 128 = 4096 tokens, random-init weights), timed end to end on the GPU: a secondary figure
     next to the headline metric."""
@@ -64,7 +64,8 @@ def model_forward(pimdl, ctx, iters=5):
     p = T.TransformerParams.bert_base(batch_size=32, seq_len=128, layer_num=12)
     model = T.Transformer(ctx, pimdl, T.synth_layers(p, ctx, pimdl, seed=1), p)
     x = torch.randn((p.n, p.token_dim), device="cuda", dtype=torch.float32)
-    model.forward(x)
+    for _ in range(3):
+        model.forward(x)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(iters):
@@ -115,8 +116,8 @@ def cpu_baseline(shapes, N, budget_s=12.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=500)
+    ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--tokens", type=int, default=8192)
     ap.add_argument("--no-model", action="store_true", help="skip the 12-layer model forward timing")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -176,8 +177,9 @@ def main():
     ms_per_step = wall_ms
 
     # per-kernel device times (HIP events on the same stream, each kernel launched on its own)
-    prof = [amms[0].profile(x1.data_ptr(), N, h.data_ptr(), warmup=3, iters=max(10, args.steps)),
-            amms[1].profile(x2.data_ptr(), N, y.data_ptr(), warmup=3, iters=max(10, args.steps))]
+    # (the engine clock takes about a hundred steps to settle after an idle period, hence the warm-up)
+    prof = [amms[0].profile(x1.data_ptr(), N, h.data_ptr(), warmup=max(3, args.warmup), iters=max(10, args.steps)),
+            amms[1].profile(x2.data_ptr(), N, y.data_ptr(), warmup=max(3, args.warmup), iters=max(10, args.steps))]
     per_amm = []
     for name, (K, vv, CC, M), p in zip(("ffn1", "ffn2"), shapes, prof):
         ab = algorithmic_bytes(N, K, vv, CC, M)

@@ -444,6 +444,22 @@ constexpr int oh_lds_bytes(int tn)
     return 256 + oh_nbuf(tn) * oh_slice_cbs(tn) * 16 * tn * 16 + oh_nbuf(tn) * OH_TOK_ITEM * (oh_slice_cbs(tn) / 2);
 }
 
+// Loads through the scalar data cache (read only) of wave-uniform addresses; they count on the
+// scalar/LDS counter, not on the vector-memory counter.
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+__device__ __forceinline__ floatx16 scalar_load16(const float* p)  // p: 4-byte aligned, wave-uniform
+{
+    floatx16 r;
+    asm volatile("s_load_dwordx16 %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(r) : "s"(p) : "memory");
+    return r;
+}
+__device__ __forceinline__ float scalar_load1(const float* p)
+{
+    float r;
+    asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(r) : "s"(p) : "memory");
+    return r;
+}
+
 // all operands of one K-step have landed; the registers pass through the asm so that no consumer
 // can be scheduled ahead of the wait
 template <int TN>
@@ -613,6 +629,11 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
 #pragma unroll
         for (int c = 0; c < TN; ++c) acc[t][c] = (v4i){0, 0, 0, 0};
 
+    // The bias values come in through scalar loads (wave-uniform addresses, the scalar counter): a
+    // vector load here would make the compiler wait on the vector-memory counter before its first
+    // use, i.e. for every output store issued so far and for the slices being prefetched, once per
+    // group of stores.  With scalar loads the epilogue contains no such wait and its stores leave
+    // back to back.
     auto epilogue = [&](uint32_t item) -> bool {
         // j and g pass through an opaque asm so that none of the address arithmetic below is
         // loop-invariant for the compiler: hoisted out of the slice loop it would occupy dozens of
@@ -626,29 +647,37 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
         const bool full = vec_store && !acc_out && tile_tok0 + OH_TOK_ITEM <= N && (colblk + 1) * WN <= M;
 #pragma unroll
         for (int c = 0; c < TN; ++c) {
-            const uint32_t f = colblk * WN + c * 16 + 4 * ge;
-            float4 bv = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (ep.bias && f < M) {
-                if (vec_store) {
-                    bv = *reinterpret_cast<const float4*>(ep.bias + f);
-                } else {
-                    bv.x = ep.bias[f];
-                    if (f + 1 < M) bv.y = ep.bias[f + 1];
-                    if (f + 2 < M) bv.z = ep.bias[f + 2];
-                    if (f + 3 < M) bv.w = ep.bias[f + 3];
-                }
+            const uint32_t f0 = colblk * WN + c * 16;  // wave-uniform
+            const uint32_t f = f0 + 4 * ge;
+            floatx16 b16;
+            if (ep.bias && f0 + 16 <= M) {
+                b16 = scalar_load16(ep.bias + f0);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) b16[e] = (ep.bias && f0 + e < M) ? scalar_load1(ep.bias + f0 + e) : 0.0f;
             }
+            float4 bv;
+            bv.x = ge == 0 ? b16[0] : ge == 1 ? b16[4] : ge == 2 ? b16[8] : b16[12];
+            bv.y = ge == 0 ? b16[1] : ge == 1 ? b16[5] : ge == 2 ? b16[9] : b16[13];
+            bv.z = ge == 0 ? b16[2] : ge == 1 ? b16[6] : ge == 2 ? b16[10] : b16[14];
+            bv.w = ge == 0 ? b16[3] : ge == 1 ? b16[7] : ge == 2 ? b16[11] : b16[15];
 #pragma unroll
             for (int t = 0; t < TM; ++t) {
                 const uint32_t tok = tok0 + t * 16 + je;
                 const v4i a = acc[t][c];
                 acc[t][c] = (v4i){0, 0, 0, 0};
-                if (tok >= N || f >= M) continue;
                 float4 o;
                 o.x = dequant(a[0], ep.scale, ep.lut_bias_term, bv.x);
                 o.y = dequant(a[1], ep.scale, ep.lut_bias_term, bv.y);
                 o.z = dequant(a[2], ep.scale, ep.lut_bias_term, bv.z);
                 o.w = dequant(a[3], ep.scale, ep.lut_bias_term, bv.w);
+                if (full) {  // workgroup-uniform: every token and column of the tile exists
+                    // streaming store: the output is not read again by this kernel
+                    typedef float v4f __attribute__((ext_vector_type(4)));
+                    __builtin_nontemporal_store((v4f){o.x, o.y, o.z, o.w}, reinterpret_cast<v4f*>(out + (size_t)tok * M + f));
+                    continue;
+                }
+                if (tok >= N || f >= M) continue;
                 if (vec_store) {  // M % 4 == 0 and f % 4 == 0: the whole float4 is in range and aligned
                     *reinterpret_cast<float4*>(out + (size_t)tok * M + f) = o;
                     if (acc_out) *reinterpret_cast<v4i*>(acc_out + (size_t)tok * M + f) = a;
