@@ -126,7 +126,7 @@ __global__ __launch_bounds__(CCS_THREADS) void ccs_kernel(const float* __restric
                                                          const float* __restrict__ cnmax,
                                                          uint8_t* __restrict__ idx, uint32_t N,
                                                          uint32_t K, uint32_t CB, uint32_t C,
-                                                         uint32_t idx_row_bytes, int vec_ok,
+                                                         uint32_t idx_row_bytes, int idx_tiled, int vec_ok,
                                                          uint32_t CB_pad, uint32_t tiles_cb,
                                                          uint32_t total_tiles)
 {
@@ -281,8 +281,13 @@ __global__ __launch_bounds__(CCS_THREADS) void ccs_kernel(const float* __restric
     // ---- packed store -----------------------------------------------------------------------
     const uint32_t tok = tok0 + lane;
     if (tok < N && cb0 < CB_pad) {
-        uint8_t* dst = idx + (size_t)tok * idx_row_bytes + (size_t)cb0 * IDX_BITS / 8;
-        if constexpr (OUT_BITS >= 128) {
+        const uint32_t byte0 = cb0 * IDX_BITS / 8;
+        uint8_t* dst = idx + idx_offset(tok, byte0, idx_row_bytes, idx_tiled);
+        if (idx_tiled && OUT_BITS >= 64) {  // one 32-bit word at a time: consecutive words are 256 bytes apart
+#pragma unroll
+            for (int w = 0; w < (OUT_BITS >= 128 ? 4 : 2); ++w)
+                *reinterpret_cast<uint32_t*>(idx + idx_offset(tok, byte0 + 4 * w, idx_row_bytes, 1)) = packed[w];
+        } else if constexpr (OUT_BITS >= 128) {
             *reinterpret_cast<uint4*>(dst) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
         } else if constexpr (OUT_BITS == 64) {
             *reinterpret_cast<uint2*>(dst) = make_uint2(packed[0], packed[1]);
@@ -404,7 +409,7 @@ __global__ __launch_bounds__(CCS_THREADS, 4) void ccs_mfma_kernel(const float* _
                                                                  const float* __restrict__ cnmax_pad,
                                                                  uint8_t* __restrict__ idx, uint32_t N,
                                                                  uint32_t K, uint32_t CB, uint32_t C,
-                                                                 uint32_t idx_row_bytes, int vec_ok,
+                                                                 uint32_t idx_row_bytes, int idx_tiled, int vec_ok,
                                                                  uint32_t tiles_cb, uint32_t total_tiles)
 {
     using S = CcsMfmaShape<V>;
@@ -582,9 +587,15 @@ __global__ __launch_bounds__(CCS_THREADS, 4) void ccs_mfma_kernel(const float* _
         __syncthreads();  // index bytes complete; every wave is done with the activation tile
         if (threadIdx.x < TT) {
             const uint32_t tok = tok0 + threadIdx.x;
-            if (tok < N)
-                *reinterpret_cast<uint2*>(idx + (size_t)tok * idx_row_bytes + tcb * (CBW / 2)) =
-                    *reinterpret_cast<const uint2*>(&ist[threadIdx.x * (CBW / 2)]);
+            if (tok < N) {
+                const uint2 w = *reinterpret_cast<const uint2*>(&ist[threadIdx.x * (CBW / 2)]);
+                if (idx_tiled) {
+                    *reinterpret_cast<uint32_t*>(idx + idx_offset(tok, tcb * (CBW / 2), idx_row_bytes, 1)) = w.x;
+                    *reinterpret_cast<uint32_t*>(idx + idx_offset(tok, tcb * (CBW / 2) + 4, idx_row_bytes, 1)) = w.y;
+                } else {
+                    *reinterpret_cast<uint2*>(idx + (size_t)tok * idx_row_bytes + tcb * (CBW / 2)) = w;
+                }
+            }
         }
     }
 }
@@ -597,7 +608,7 @@ __global__ __launch_bounds__(256) void ccs_generic_kernel(const float* __restric
                                                          uint8_t* __restrict__ idx, uint32_t N,
                                                          uint32_t K, uint32_t v, uint32_t CB,
                                                          uint32_t CB_pad, uint32_t C,
-                                                         uint32_t idx_row_bytes)
+                                                         uint32_t idx_row_bytes, int idx_tiled)
 {
     // a lane produces one whole output byte (two codebooks when IDX_BITS == 4)
     constexpr int CB_PER_BYTE = 8 / IDX_BITS;
@@ -627,19 +638,19 @@ __global__ __launch_bounds__(256) void ccs_generic_kernel(const float* __restric
         }
         outv |= bi << (IDX_BITS * h);
     }
-    idx[(size_t)tok * idx_row_bytes + byte] = (uint8_t)outv;
+    idx[idx_offset(tok, byte, idx_row_bytes, idx_tiled)] = (uint8_t)outv;
 }
 
 // packed indices -> uint16 at the reference's tiled offset (index_calc_host.cpp:41-49)
 template <int IDX_BITS>
 __global__ void unpack_idx_kernel(const uint8_t* __restrict__ idx, uint16_t* __restrict__ out,
-                                  uint32_t N, uint32_t CB, uint32_t idx_row_bytes, uint32_t n_stile,
-                                  uint32_t cb_mtile)
+                                  uint32_t N, uint32_t CB, uint32_t idx_row_bytes, int idx_tiled,
+                                  uint32_t n_stile, uint32_t cb_mtile)
 {
     const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (gid >= (uint64_t)N * CB) return;
     const uint32_t n = gid / CB, cb = gid % CB;
-    const uint8_t b = idx[(size_t)n * idx_row_bytes + (size_t)cb * IDX_BITS / 8];
+    const uint8_t b = idx[idx_offset(n, cb * IDX_BITS / 8, idx_row_bytes, idx_tiled)];
     const uint16_t val = (IDX_BITS == 4) ? ((b >> (4 * (cb & 1))) & 0xF) : b;
     const uint64_t off = (uint64_t)(n / n_stile) * n_stile * CB + (uint64_t)(cb / cb_mtile) * n_stile * cb_mtile +
                          (uint64_t)(n % n_stile) * cb_mtile + (cb % cb_mtile);
@@ -649,7 +660,8 @@ __global__ void unpack_idx_kernel(const uint8_t* __restrict__ idx, uint16_t* __r
 // uint16 centroid ids at the reference's tiled offset -> packed rows (padded codebooks get index 0)
 template <int IDX_BITS>
 __global__ void pack_idx_kernel(const uint16_t* __restrict__ in, uint8_t* __restrict__ idx, uint32_t N,
-                                uint32_t CB, uint32_t idx_row_bytes, uint32_t n_stile, uint32_t cb_mtile)
+                                uint32_t CB, uint32_t idx_row_bytes, int idx_tiled, uint32_t n_stile,
+                                uint32_t cb_mtile)
 {
     constexpr int CB_PER_BYTE = 8 / IDX_BITS;
     const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -664,7 +676,7 @@ __global__ void pack_idx_kernel(const uint16_t* __restrict__ in, uint8_t* __rest
             outv |= (uint32_t)(in[off] & ((1u << IDX_BITS) - 1)) << (IDX_BITS * h);
         }
     }
-    idx[gid] = (uint8_t)outv;
+    idx[idx_offset(n, byte, idx_row_bytes, idx_tiled)] = (uint8_t)outv;
 }
 
 template <int V, int IDX_BITS>
@@ -688,10 +700,10 @@ int launch_ccs_t(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_ce
     const float* cnmax = aux + ccs_aux_floats(g);
     if (ccs_exact_only())
         hipLaunchKernelGGL((ccs_kernel<V, IDX_BITS, false>), grid, dim3(CCS_THREADS), 0, ctx->stream, d_x, d_cent,
-                           aux, cnmax, d_idx, n, g.K, g.CB, g.C, g.idx_row_bytes, vec_ok, g.CB_pad, tiles_cb, total);
+                           aux, cnmax, d_idx, n, g.K, g.CB, g.C, g.idx_row_bytes, (int)g.idx_tiled, vec_ok, g.CB_pad, tiles_cb, total);
     else
         hipLaunchKernelGGL((ccs_kernel<V, IDX_BITS, true>), grid, dim3(CCS_THREADS), 0, ctx->stream, d_x, d_cent,
-                           aux, cnmax, d_idx, n, g.K, g.CB, g.C, g.idx_row_bytes, vec_ok, g.CB_pad, tiles_cb, total);
+                           aux, cnmax, d_idx, n, g.K, g.CB, g.C, g.idx_row_bytes, (int)g.idx_tiled, vec_ok, g.CB_pad, tiles_cb, total);
     return hip_check(ctx, hipGetLastError(), "ccs_kernel launch");
 }
 
@@ -718,7 +730,7 @@ int launch_ccs_mfma(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d
     const float* aux_a = cnmax + g.CB;
     const float* cnmax_pad = aux_a + (size_t)(g.CB_pad / 2) * (g.v + 1) * 64;
     hipLaunchKernelGGL((ccs_mfma_kernel<V>), grid, dim3(CCS_THREADS), 0, ctx->stream, d_x, d_cent, aux_a, cnmax_pad,
-                       d_idx, n, g.K, g.CB, g.C, g.idx_row_bytes, vec_ok, tiles_cb, total);
+                       d_idx, n, g.K, g.CB, g.C, g.idx_row_bytes, (int)g.idx_tiled, vec_ok, tiles_cb, total);
     return hip_check(ctx, hipGetLastError(), "ccs_mfma_kernel launch");
 }
 
@@ -743,7 +755,7 @@ int launch_ccs_bits(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d
             const uint64_t total = (uint64_t)n * (g.CB_pad / (8 / IDX_BITS));
             dim3 grid((uint32_t)((total + 255) / 256));
             hipLaunchKernelGGL((ccs_generic_kernel<IDX_BITS>), grid, dim3(256), 0, ctx->stream, d_x, d_cent, d_idx,
-                               n, g.K, g.v, g.CB, g.CB_pad, g.C, g.idx_row_bytes);
+                               n, g.K, g.v, g.CB, g.CB_pad, g.C, g.idx_row_bytes, (int)g.idx_tiled);
             return hip_check(ctx, hipGetLastError(), "ccs_generic_kernel launch");
         }
     }
@@ -808,10 +820,10 @@ int launch_unpack_idx(Ctx* ctx, const AmmGeom& g, const uint8_t* d_idx, uint16_t
     dim3 grid((uint32_t)((total + 255) / 256));
     if (g.idx_bits == 4)
         hipLaunchKernelGGL((unpack_idx_kernel<4>), grid, dim3(256), 0, ctx->stream, d_idx, d_idx16, n, g.CB,
-                           g.idx_row_bytes, n_stile, cb_mtile);
+                           g.idx_row_bytes, (int)g.idx_tiled, n_stile, cb_mtile);
     else
         hipLaunchKernelGGL((unpack_idx_kernel<8>), grid, dim3(256), 0, ctx->stream, d_idx, d_idx16, n, g.CB,
-                           g.idx_row_bytes, n_stile, cb_mtile);
+                           g.idx_row_bytes, (int)g.idx_tiled, n_stile, cb_mtile);
     return hip_check(ctx, hipGetLastError(), "unpack_idx_kernel launch");
 }
 
@@ -823,10 +835,10 @@ int launch_pack_idx(Ctx* ctx, const AmmGeom& g, const uint16_t* d_idx16, uint8_t
     dim3 grid((uint32_t)((total + 255) / 256));
     if (g.idx_bits == 4)
         hipLaunchKernelGGL((pack_idx_kernel<4>), grid, dim3(256), 0, ctx->stream, d_idx16, d_idx, n, g.CB,
-                           g.idx_row_bytes, n_stile, cb_mtile);
+                           g.idx_row_bytes, (int)g.idx_tiled, n_stile, cb_mtile);
     else
         hipLaunchKernelGGL((pack_idx_kernel<8>), grid, dim3(256), 0, ctx->stream, d_idx16, d_idx, n, g.CB,
-                           g.idx_row_bytes, n_stile, cb_mtile);
+                           g.idx_row_bytes, (int)g.idx_tiled, n_stile, cb_mtile);
     return hip_check(ctx, hipGetLastError(), "pack_idx_kernel launch");
 }
 

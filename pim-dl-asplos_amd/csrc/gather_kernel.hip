@@ -536,16 +536,19 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
     uint32_t lut_item = blockIdx.x, lut_s = 0, ix_item = blockIdx.x, ix_s = 0;
     const int8_t* dma_base;   // uniform: start of the slice at the LUT stream position
     const uint32_t dma_lane = wave * 1024 + lane * 16;
-    const uint8_t* ix_base;   // uniform: idx + byte offset of the slice inside a row
-    uint32_t ix_lane_off;     // per lane: token row offset (rows of one workgroup tile span < 4 GB: checked at launch)
+    const uint8_t* ix_base;   // uniform: the 256-byte block of index words at the index stream position
+    uint32_t ix_lane_off;     // per lane: its token's word inside a block
     auto locate_lut = [&]() {
         dma_base = lut + (size_t)(lut_item / n_token_tiles) * CB_pad * (WN * 16);
     };
+    // Index words live as [N/64][row words][64 tokens]: the word of a slice for this wave's 64 tokens
+    // is one contiguous 256-byte block (see idx_offset).
+    const uint32_t last_block = (N - 1) / 64;
     auto locate_ix = [&]() {
-        uint32_t tok = (ix_item % n_token_tiles) * OH_TOK_ITEM + wave * 64 + lane;
-        if (tok >= N) tok = N - 1;  // clamp: results of such tokens are never stored
-        ix_base = idx;
-        ix_lane_off = tok * idx_row_bytes;
+        uint32_t blk = (ix_item % n_token_tiles) * (OH_TOK_ITEM / 64) + wave;
+        if (blk > last_block) blk = last_block;  // clamp: results of such tokens are never stored
+        ix_base = idx + (size_t)blk * idx_row_bytes * 64;
+        ix_lane_off = lane * 4;
     };
     // real = false (past the end of the stream): the operation re-copies the first slice of the
     // LUT into a buffer nobody reads any more, so that every slice issues the same number of
@@ -574,12 +577,12 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
     auto ix_op = [&](uint32_t ibuf, bool real, auto ic) {
         constexpr int i = decltype(ic)::value;
         const uint32_t dst = IBUF0 + ibuf * IBYTES + wave * IWAVE;  // wave-uniform; lanes add 4*lane
-        const uint8_t* src = real ? ix_base + 4 * i : idx;  // uniform
+        const uint8_t* src = real ? ix_base + 256 * i : idx;  // uniform
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + (real ? ix_lane_off : 0u)),
                                          (__attribute__((address_space(3))) void*)(smem + dst + 256 * i), 4, 0, 0);
     };
     auto ix_advance = [&]() {
-        ix_base += G / 2;
+        ix_base += (G / 8) * 256;
         if (++ix_s == nslices) {
             ix_s = 0;
             ix_item += gridDim.x;
@@ -1048,9 +1051,8 @@ bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::s
     g->idx_row_bytes = g->CB_pad * g->idx_bits / 8;
     const bool i8 = d.lut_dtype == PIMDL_LUT_I8;
     g->q = ct >= 128 ? 2 : 4;
-    // the one-hot kernel addresses index rows with 32-bit offsets
-    const bool idx_fits = (uint64_t)d.max_n * g->idx_row_bytes <= 0xFFFFFFFFull;
-    g->gather_kind = (i8 && C <= 16 && idx_fits && !gather_rows_only()) ? 1 : 0;
+    g->gather_kind = (i8 && C <= 16 && !gather_rows_only()) ? 1 : 0;
+    g->idx_tiled = g->gather_kind == 1;
     if (g->gather_kind == 1) {
         // One-hot matrix-core kernel: an item is 256 tokens x 16*TN columns, all items cost the
         // same.  Take the TN that fills the persistent grid (two workgroups per CU) most evenly for

@@ -346,7 +346,7 @@ int pimdl_amm_run(pimdl_amm* a, const float* in, uint32_t n, float* out)
     bool out_host;
     if ((rc = stage_input(ctx, a->g, in, n, &d_in))) return rc;
     if ((rc = stage_output(ctx, a->g, out, n, &d_out, &out_host))) return rc;
-    if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, (size_t)n * a->g.idx_row_bytes, "hipMalloc(index scratch)"))) return rc;
+    if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, idx_buffer_bytes(a->g, n), "hipMalloc(index scratch)"))) return rc;
     if ((rc = launch_ccs(ctx, a->g, d_in, a->d_centroids, ctx->d_idx, n))) return rc;
     if ((rc = launch_gather(ctx, *a, ctx->d_idx, d_out, nullptr, n))) return rc;
     return finish_output(ctx, a->g, out, n, out_host);
@@ -365,7 +365,7 @@ int pimdl_amm_run_debug(pimdl_amm* a, const float* in, uint32_t n, float* out, u
     bool out_host;
     if ((rc = stage_input(ctx, g, in, n, &d_in))) return rc;
     if ((rc = stage_output(ctx, g, out, n, &d_out, &out_host))) return rc;
-    if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, (size_t)n * g.idx_row_bytes, "hipMalloc(index scratch)"))) return rc;
+    if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, idx_buffer_bytes(g, n), "hipMalloc(index scratch)"))) return rc;
     if (acc_out && (rc = ensure(ctx, &ctx->d_acc, &ctx->acc_bytes, (size_t)n * g.M * 4, "hipMalloc(acc scratch)"))) return rc;
     if (idx_out && (rc = ensure(ctx, &ctx->d_idx16, &ctx->idx16_bytes, (size_t)n * g.CB * 2, "hipMalloc(idx16 scratch)"))) return rc;
     if ((rc = launch_ccs(ctx, g, d_in, a->d_centroids, ctx->d_idx, n))) return rc;
@@ -390,7 +390,7 @@ int pimdl_amm_profile(pimdl_amm* a, const float* in_dev, uint32_t n, float* out_
     if (!timing || !iters || !n) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_profile: bad arguments");
     if (!is_device_ptr(in_dev) || !is_device_ptr(out_dev))
         return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_profile: in/out must be device pointers");
-    if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, (size_t)n * a->g.idx_row_bytes, "hipMalloc(index scratch)"))) return rc;
+    if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, idx_buffer_bytes(a->g, n), "hipMalloc(index scratch)"))) return rc;
     for (uint32_t i = 0; i < warmup; ++i) {
         if ((rc = launch_ccs(ctx, a->g, in_dev, a->d_centroids, ctx->d_idx, n))) return rc;
         if ((rc = launch_gather(ctx, *a, ctx->d_idx, out_dev, nullptr, n))) return rc;
@@ -423,7 +423,7 @@ static int index_calc_common(Ctx* ctx, const AmmGeom& g, const float* in, const 
     int rc;
     const float* d_in;
     if ((rc = stage_input(ctx, g, in, n, &d_in))) return rc;
-    if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, (size_t)n * g.idx_row_bytes, "hipMalloc(index scratch)"))) return rc;
+    if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, idx_buffer_bytes(g, n), "hipMalloc(index scratch)"))) return rc;
     if ((rc = ensure(ctx, &ctx->d_idx16, &ctx->idx16_bytes, (size_t)n * g.CB * 2, "hipMalloc(idx16 scratch)"))) return rc;
     if ((rc = launch_ccs(ctx, g, d_in, d_cent, ctx->d_idx, n))) return rc;
     if ((rc = launch_unpack_idx(ctx, g, ctx->d_idx, ctx->d_idx16, n, n_stile_size, cb_mtile_size))) return rc;
@@ -507,7 +507,7 @@ int pimdl_amm_run_tiled(pimdl_amm* a, const float* in, uint32_t n, float* out, c
     if ((rc = resolve_tiling(ctx, a->g, n, tiling, &til, &ident))) return rc;
     const float* d_in;
     if ((rc = stage_input(ctx, a->g, in, n, &d_in))) return rc;
-    if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, (size_t)n * a->g.idx_row_bytes, "hipMalloc(index scratch)"))) return rc;
+    if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, idx_buffer_bytes(a->g, n), "hipMalloc(index scratch)"))) return rc;
     if ((rc = launch_ccs(ctx, a->g, d_in, a->d_centroids, ctx->d_idx, n))) return rc;
     return gather_to(a, n, out, til, ident);
 }
@@ -521,7 +521,7 @@ int pimdl_lut_gather_tiled(pimdl_amm* a, const uint16_t* idx, uint32_t n, float*
     pimdl_tiling til;
     bool ident;
     if ((rc = resolve_tiling(ctx, g, n, tiling, &til, &ident))) return rc;
-    if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, (size_t)n * g.idx_row_bytes, "hipMalloc(index scratch)"))) return rc;
+    if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, idx_buffer_bytes(g, n), "hipMalloc(index scratch)"))) return rc;
     if ((rc = ensure(ctx, &ctx->d_idx16, &ctx->idx16_bytes, (size_t)n * g.CB * 2, "hipMalloc(idx16 scratch)"))) return rc;
     if ((rc = hip_check(ctx, hipMemcpyAsync(ctx->d_idx16, idx, (size_t)n * g.CB * 2, hipMemcpyHostToDevice, ctx->stream), "H2D idx"))) return rc;
     if ((rc = launch_pack_idx(ctx, g, ctx->d_idx16, ctx->d_idx, n, til.n_stile_size, til.cb_mtile_size))) return rc;

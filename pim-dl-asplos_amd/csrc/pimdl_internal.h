@@ -14,6 +14,10 @@ namespace pimdl {
 //
 // Index rows   [N][idx_row_bytes] bytes; IDX_BITS = 4 (C <= 16, codebook 2k in the low nibble
 //              of byte k) or 8.  Codebooks are padded to a multiple of 32 with index 0.
+//              idx_tiled (operators served by the one-hot gather): the same bytes stored as
+//              [N/64][idx_row_bytes/4][64 tokens][4 bytes], so that the 32-bit index words one
+//              wave needs for one codebook slice (64 tokens x 1 word) are 256 contiguous bytes;
+//              the buffer covers N rounded up to 64 tokens.
 // int8 LUT     gather_kind 0: tiled [M_pad / col_block][CB_pad][C_tile][col_block] bytes
 //              (col_block = 16*Q); gather_kind 1: [M_pad / col_block][CB_pad][col_block][16] bytes
 //              (the 16 centroid entries of a column are contiguous).  Either way one (column block,
@@ -24,6 +28,7 @@ namespace pimdl {
 struct AmmGeom {
     uint32_t K, v, CB, CB_pad, C, C_tile, M, M_pad;
     uint32_t idx_bits, idx_row_bytes;
+    uint32_t idx_tiled;     // layout of the packed index buffer, see above
     // gather kernel
     uint32_t gather_kind;   // 0: byte-adder rows kernel, 1: one-hot matrix-core kernel (int8, C <= 16)
     uint32_t q;             // 16-byte chunks per LUT row in LDS
@@ -35,6 +40,21 @@ struct AmmGeom {
     // ccs kernel
     uint32_t ccs_row_floats, ccs_cb_per_wg, ccs_lds_bytes;
 };
+
+// bytes of a packed index buffer for n tokens
+inline size_t idx_buffer_bytes(const AmmGeom& g, uint32_t n)
+{
+    return (size_t)(g.idx_tiled ? (n + 63) / 64 * 64 : n) * g.idx_row_bytes;
+}
+
+#ifdef __HIPCC__
+// byte offset of byte `byte` of token `tok`'s index row (aligned groups of 4 bytes stay contiguous)
+__device__ __forceinline__ size_t idx_offset(uint32_t tok, uint32_t byte, uint32_t row_bytes, int tiled)
+{
+    return tiled ? ((size_t)(tok >> 6) * (row_bytes >> 2) + (byte >> 2)) * 256 + ((tok & 63) << 2) + (byte & 3)
+                 : (size_t)tok * row_bytes + byte;
+}
+#endif
 
 struct Ctx;
 
