@@ -69,6 +69,19 @@ inline size_t ccs_aux_a_floats(const AmmGeom& g)
     return (size_t)(g.CB_pad / 2) * (g.v + 1) * 64 + g.CB_pad;  // A-operand images, padded cnmax
 }
 
+// bf16-split search (v = 4, C <= 16): offset in floats of its operands behind everything else, and
+// their size.  The offset is rounded up to 16 bytes (uint4 operand images).
+inline bool ccs_has_bf16(const AmmGeom& g) { return g.v == 4 && g.C <= 16; }
+inline size_t ccs_bf16_offset(const AmmGeom& g)
+{
+    const size_t o = (size_t)g.CB * g.C * g.v + ccs_aux_floats(g) + g.CB + ccs_aux_a_floats(g);
+    return (o + 3) / 4 * 4;
+}
+inline size_t ccs_bf16_floats(const AmmGeom& g)
+{
+    return ccs_has_bf16(g) ? (size_t)(g.CB_pad / 2) * 3 * 64 * 4 + (size_t)g.CB_pad * 16 : 0;
+}
+
 template <int N, typename F>
 __device__ __forceinline__ void static_for(F&& f)
 {
@@ -600,6 +613,307 @@ __global__ __launch_bounds__(CCS_THREADS, 4) void ccs_mfma_kernel(const float* _
     }
 }
 
+// =============================================================================================
+// bf16-split variant of the MFMA search for v = 4 (C <= 16).  The fp32 MFMA above shares the fp32
+// units with the VALU, so its five instructions per item (147 ns) add to the ~50 VALU operations of
+// the top-two search (100 ns).  v_mfma_f32_32x32x16_bf16 is twice as fast per K-slot and runs beside
+// VALU work.  bf16 has 8 significand bits, so each fp32 value is cut into three bf16 pieces and six
+// of the nine cross products are kept (see `scores` below); the score then carries a known error
+// bound like the fp32 form's, only larger (A2 below), and everything after the scores -- tagged
+// keys, tournament, margin test, exact replay -- is the same.  Operands:
+//   aux_b [CB_pad/2 pairs][3][64 lanes] uint4  A-operand images (bf16 pieces of -2c, by K-slot)
+//   cn16  [CB_pad][16] float                   |c|^2 (r for padded codebooks, 3e38 for ids past C)
+// =============================================================================================
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+// K-slot register rho (0..11, four per MFMA) of lane (row i, half kh) pairs dims 2kh, 2kh+1 of codebook
+// rho / 6 of the pair with piece  {ch, cm, ch, cm, cl, ch}[rho % 6]  of -2c; the search kernel supplies
+// {xh, xh, xm, xm, xh, xl} in the same registers.  Rows of the other codebook hold zeros there.
+__global__ void ccs_prep_bf16_kernel(const float* __restrict__ cent, uint4* __restrict__ aux_b,
+                                     float* __restrict__ cn16, uint32_t CB, uint32_t C)
+{
+    constexpr uint32_t v = 4;
+    const uint32_t pair = blockIdx.x, lane = threadIdx.x;
+    const uint32_t i = lane & 31, kh = lane >> 5;
+    const uint32_t h = (i >> 2) & 1, r = (i & 3) + 4 * (i >> 3);
+    const uint32_t cb = 2 * pair + h;
+    const bool real = (cb < CB) && (r < C);
+    const float* cp = cent + ((size_t)cb * C + r) * v;
+    uint32_t piece[3] = {0, 0, 0};  // (dim 2kh | dim 2kh+1 << 16) of ch, cm, cl
+    if (real) {
+        uint32_t pc[2][3];
+        for (int d = 0; d < 2; ++d) {
+            const float a = -2.0f * cp[2 * kh + d];
+            const uint32_t au = __float_as_uint(a);
+            const float r1 = __fsub_rn(a, __uint_as_float(au & 0xffff0000u));
+            const uint32_t r1u = __float_as_uint(r1);
+            const float r2 = __fsub_rn(r1, __uint_as_float(r1u & 0xffff0000u));
+            pc[d][0] = au >> 16;
+            pc[d][1] = r1u >> 16;
+            pc[d][2] = __float_as_uint(r2) >> 16;
+        }
+        for (int t = 0; t < 3; ++t) piece[t] = pc[0][t] | (pc[1][t] << 16);
+    }
+    const int term[6] = {0, 1, 0, 1, 2, 0};
+    for (uint32_t m = 0; m < 3; ++m) {
+        uint32_t w[4];
+        for (uint32_t q = 0; q < 4; ++q) {
+            const uint32_t rho = 4 * m + q;
+            w[q] = (rho / 6 == h) ? piece[term[rho % 6]] : 0u;
+        }
+        aux_b[((size_t)pair * 3 + m) * 64 + lane] = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+    if (kh == 0) {
+        float cn = (float)r;  // a padded codebook scores r against centroid r: index 0 with a margin of 1
+        if (real) {
+            cn = 0.0f;
+            for (uint32_t t = 0; t < v; ++t) cn = fmaf(cp[t], cp[t], cn);
+        } else if (cb < CB) {
+            cn = 3e38f;  // centroid ids past C never win
+        }
+        cn16[(size_t)(2 * pair + h) * 16 + r] = cn;
+    }
+}
+
+__global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* __restrict__ x,
+                                                                 const float* __restrict__ cent,
+                                                                 const uint4* __restrict__ aux_b,
+                                                                 const float* __restrict__ cn16,
+                                                                 const float* __restrict__ cnmax_pad,
+                                                                 uint8_t* __restrict__ idx, uint32_t N,
+                                                                 uint32_t K, uint32_t CB, uint32_t C,
+                                                                 uint32_t idx_row_bytes, int idx_tiled, int vec_ok,
+                                                                 uint32_t tiles_cb, uint32_t total_tiles)
+{
+    constexpr int V = 4;
+    using S = CcsMfmaShape<V>;
+    constexpr int TF = S::TF, PITCH = S::PITCH, TT = S::TILE_TOKENS, CBW = S::CBW, TG = S::TG;
+    constexpr int NM = 3;  // MFMAs per item: 2 codebooks x 4 dims x 6 cross terms = 48 K-slots
+    constexpr int ITEMS = S::ITEMS;
+    __shared__ __attribute__((aligned(16))) float tile[S::X_FLOATS];
+    __shared__ __attribute__((aligned(16))) float cst[S::CENT_FLOATS];
+    __shared__ __attribute__((aligned(16))) uint8_t ist[TT * (CBW / 2)];
+    __shared__ __attribute__((aligned(16))) float cnl[CBW * 16];  // |c|^2 of the tile's centroids: the accumulators start from them
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t j = lane & 31, h = lane >> 5;  // token within a group, codebook of the pair
+
+    constexpr int F4_PER_ROW = TF / 4;
+    constexpr int ROWS_PER_PASS = CCS_THREADS / F4_PER_ROW;
+    constexpr int PASSES = TT / ROWS_PER_PASS;
+    static_assert(CCS_THREADS % F4_PER_ROW == 0 && TT % ROWS_PER_PASS == 0, "tile shape");
+    const uint32_t fq = threadIdx.x % F4_PER_ROW;
+    const uint32_t fr0 = threadIdx.x / F4_PER_ROW;
+    auto fetch = [&](float4 (&pf)[PASSES], uint32_t tile_id) {
+        const uint32_t t_tok0 = (tile_id / tiles_cb) * TT;
+        const uint32_t col = (tile_id % tiles_cb) * TF + 4 * fq;
+#pragma unroll
+        for (int i = 0; i < PASSES; ++i) {
+            uint32_t tok = t_tok0 + fr0 + i * ROWS_PER_PASS;
+            if (tok >= N) tok = N - 1;  // rows past N repeat the last token; never stored
+            const float* src = x + (size_t)tok * K + col;
+            if (vec_ok && col + 4 <= K) {
+                pf[i] = *reinterpret_cast<const float4*>(src);
+            } else {
+                pf[i].x = (col + 0 < K) ? src[0] : 0.0f;
+                pf[i].y = (col + 1 < K) ? src[1] : 0.0f;
+                pf[i].z = (col + 2 < K) ? src[2] : 0.0f;
+                pf[i].w = (col + 3 < K) ? src[3] : 0.0f;
+            }
+        }
+    };
+    // operands of this lane inside the tile: row of token (32 tg + j), columns of pair (2 wave + pl)
+    const float* brow0 = tile + j * PITCH + 2 * wave * 2 * V;
+
+    float4 pf[PASSES];
+    if (blockIdx.x < total_tiles) fetch(pf, blockIdx.x);
+
+    for (uint32_t tile_id = blockIdx.x; tile_id < total_tiles; tile_id += gridDim.x) {
+        const uint32_t tok0 = (tile_id / tiles_cb) * TT;
+        const uint32_t tcb = tile_id % tiles_cb;          // codebooks 16 tcb .. 16 tcb + 15
+        const uint32_t pair0 = tcb * (CBW / 2) + 2 * wave;  // first of this wave's two pairs
+
+        uint4 aq[2][NM];
+#pragma unroll
+        for (int pl = 0; pl < 2; ++pl)
+#pragma unroll
+            for (int m = 0; m < NM; ++m) aq[pl][m] = aux_b[((size_t)(pair0 + pl) * NM + m) * 64 + lane];
+        // every global load the search needs is issued here, ahead of the next tile's prefetch:
+        // loads complete in order, so a later load would have to wait for the prefetch from HBM
+        float cmax[2];
+#pragma unroll
+        for (int pl = 0; pl < 2; ++pl) cmax[pl] = cnmax_pad[2 * (pair0 + pl) + h];
+        // raw centroids of the tile's codebooks, only read by exact replays
+        const uint32_t cb_here = (CB - tcb * CBW < (uint32_t)CBW) ? CB - tcb * CBW : (uint32_t)CBW;
+        const uint32_t cent_fl = cb_here * C * V;
+        const float* csrc = cent + (size_t)tcb * CBW * C * V;  // 16-byte aligned: CBW * V * 4 bytes per c
+#pragma unroll
+        for (int i = 0; i < PASSES; ++i)
+            *reinterpret_cast<float4*>(&tile[(fr0 + i * ROWS_PER_PASS) * PITCH + 4 * fq]) = pf[i];
+        for (uint32_t i = threadIdx.x; i < cent_fl / 4; i += CCS_THREADS)
+            reinterpret_cast<float4*>(cst)[i] = reinterpret_cast<const float4*>(csrc)[i];
+        if (threadIdx.x < cent_fl % 4) cst[cent_fl - 1 - threadIdx.x] = csrc[cent_fl - 1 - threadIdx.x];
+        if (threadIdx.x < CBW * 16 / 4)
+            reinterpret_cast<float4*>(cnl)[threadIdx.x] = reinterpret_cast<const float4*>(cn16 + (size_t)tcb * CBW * 16)[threadIdx.x];
+        __syncthreads();
+        if (tile_id + gridDim.x < total_tiles) fetch(pf, tile_id + gridDim.x);
+
+        // Scores of item `it` (pair pl, token group tg) for this lane's token: this lane (half h) holds
+        // dims 2h, 2h+1 of both codebooks of the pair.  Each value is cut into three bf16 pieces by
+        // masking (x = xh + xm + xl exactly: 8 + 8 + 8 significand bits); the A operand holds the same
+        // pieces of -2c, and the K-slots pair them as  xh*ch, xh*cm, xm*ch, xm*cm, xh*cl, xl*ch  (the three
+        // omitted products are below 2^-20 |x||c|).  Products of bf16 values are exact in fp32; the
+        // accumulators start from |c|^2.  xx_out: |x|^2 over the lane's own codebook (for the bound).
+        auto scores = [&](floatx16& acc, float& xx_out, int it) {
+            const int pl = it / TG, tg = it % TG;
+            const float* brow = brow0 + tg * 32 * PITCH + pl * 2 * V;
+            const float2 x0 = *reinterpret_cast<const float2*>(brow + 2 * h);      // codebook 0 of the pair
+            const float2 x1 = *reinterpret_cast<const float2*>(brow + V + 2 * h);  // codebook 1
+            const float4* cnp = reinterpret_cast<const float4*>(cnl + (2 * (2 * wave + pl) + h) * 16);
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+                const float4 c4 = cnp[q4];
+                acc[4 * q4 + 0] = c4.x;
+                acc[4 * q4 + 1] = c4.y;
+                acc[4 * q4 + 2] = c4.z;
+                acc[4 * q4 + 3] = c4.w;
+            }
+            uint32_t H[2], Mm[2], L[2];
+            float part[2];
+#pragma unroll
+            for (int cbh = 0; cbh < 2; ++cbh) {
+                const float a = cbh ? x1.x : x0.x, b = cbh ? x1.y : x0.y;
+                const uint32_t au = __float_as_uint(a), bu = __float_as_uint(b);
+                const float ar1 = a - __uint_as_float(au & 0xffff0000u), br1 = b - __uint_as_float(bu & 0xffff0000u);
+                const uint32_t ar1u = __float_as_uint(ar1), br1u = __float_as_uint(br1);
+                const float ar2 = ar1 - __uint_as_float(ar1u & 0xffff0000u), br2 = br1 - __uint_as_float(br1u & 0xffff0000u);
+                H[cbh] = __builtin_amdgcn_perm(bu, au, 0x07060302u);       // (bf16 of dim 2h | bf16 of dim 2h+1 << 16)
+                Mm[cbh] = __builtin_amdgcn_perm(br1u, ar1u, 0x07060302u);
+                L[cbh] = __builtin_amdgcn_perm(__float_as_uint(br2), __float_as_uint(ar2), 0x07060302u);
+                part[cbh] = fmaf(b, b, a * a);
+            }
+            // |x|^2 of codebook h: lanes l and l+32 each hold half of it for both codebooks
+            const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(part[0]), __float_as_uint(part[1]), false, false);
+            xx_out = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+            const uint4 b0 = make_uint4(H[0], H[0], Mm[0], Mm[0]);
+            const uint4 b1 = make_uint4(H[0], L[0], H[1], H[1]);
+            const uint4 b2 = make_uint4(Mm[1], Mm[1], H[1], L[1]);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, aq[pl][0]), __builtin_bit_cast(bf16x8, b0), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, aq[pl][1]), __builtin_bit_cast(bf16x8, b1), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, aq[pl][2]), __builtin_bit_cast(bf16x8, b2), acc, 0, 0, 0);
+        };
+
+        // words[tg / 2], 16 bits per token group: nibble of (pair pl, half h) at bit 8 pl + 4 h
+        uint32_t words[TG / 2];
+#pragma unroll
+        for (int i = 0; i < TG / 2; ++i) words[i] = 0;
+        uint32_t need = 0;  // bit it: item it must be replayed exactly by this lane
+
+        floatx16 acc_cur, acc_nxt;
+        float xx_cur, xx_nxt;
+        scores(acc_cur, xx_cur, 0);
+        static_for<ITEMS>([&](auto itc) {
+            constexpr int it = decltype(itc)::value;
+            constexpr int pl = it / TG, tg = it % TG;
+            (void)tg;
+            if constexpr (it + 1 < ITEMS) scores(acc_nxt, xx_nxt, it + 1);
+            const float xx = xx_cur;
+            // smallest (m1) and second smallest (m2) of the 16 id-tagged scores, 36 VALU operations:
+            // five triples give (min3, med3) each; the overall second smallest is the smaller of
+            // the second smallest of the six group minima and the smallest of the group medians.
+            float key[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                key[r] = __uint_as_float((__float_as_uint(acc_cur[r]) & ~15u) | (uint32_t)r);
+            float lo[5], md[5];
+#pragma unroll
+            for (int i = 0; i < 5; ++i) {
+                lo[i] = vmin3(key[3 * i], key[3 * i + 1], key[3 * i + 2]);
+                md[i] = __builtin_amdgcn_fmed3f(key[3 * i], key[3 * i + 1], key[3 * i + 2]);
+            }
+            const float a1 = vmin3(lo[0], lo[1], lo[2]), a2 = __builtin_amdgcn_fmed3f(lo[0], lo[1], lo[2]);
+            const float b1 = vmin3(lo[3], lo[4], key[15]), b2 = __builtin_amdgcn_fmed3f(lo[3], lo[4], key[15]);
+            const float m1 = vmin(a1, b1);
+            const float m2 = vmin3(vmin3(md[0], md[1], md[2]), vmin3(md[3], md[4], vmax(a1, b1)), vmin(a2, b2));
+            const uint32_t bi = __float_as_uint(m1) & 15u;
+            const float mag = xx + cmax[pl];
+            // 2 * [ (v+1)u (|c|^2) + 16u (omitted products) + 103u (51 additions, each within u of a partial
+            //       sum below 2.02 mag) + 2(v+2)u (the reference's own chain) ] = 2 * 136u
+            constexpr float A2 = 2.0f * 136.0f * 5.9604645e-8f;
+            constexpr float B2 = 2.0f * 16.0f * 2.3841858e-7f;               // 2 * 2^(4-22)
+            const float thr = fmaf(A2, mag, fmaf(B2, fabsf(m2), 1.001e-6f));
+            // NaN anywhere makes a compare false, which counts as "not safe"
+            const bool safe = ((m2 - m1) > thr) && (mag < 1e36f);
+            need |= (safe ? 0u : 1u) << it;
+            words[tg / 2] |= bi << (16 * (tg % 2) + 8 * pl + 4 * h);
+            if constexpr (it + 1 < ITEMS) {
+                acc_cur = acc_nxt;
+                xx_cur = xx_nxt;
+            }
+        });
+
+        // ---- exact replay of the items that failed the margin test (rare, lane-divergent) -------
+        if (__builtin_amdgcn_ballot_w64(need != 0) != 0) {
+            // kept rolled on purpose: the replay is rare and must not cost the fast path registers
+#pragma nounroll
+            for (int it = 0; it < ITEMS; ++it) {
+                if (!((need >> it) & 1u)) continue;
+                const int pl = it / TG, tg = it % TG;
+                const uint32_t cbl = 2 * (2 * wave + pl) + h;
+                uint32_t bi = 0;
+                if (tcb * CBW + cbl < CB) {
+                    const float* xo = brow0 + tg * 32 * PITCH + pl * 2 * V + V * h;
+                    const float* cp = cst + cbl * C * V;
+                    float best = 0.0f;
+#pragma nounroll
+                    for (uint32_t c = 0; c < C; ++c) {
+                        float diff = __fsub_rn(xo[0], cp[c * V + 0]);
+                        float d = __fmul_rn(diff, diff);
+#pragma unroll
+                        for (int t = 1; t < V; ++t) {
+                            diff = __fsub_rn(xo[t], cp[c * V + t]);
+                            d = __fadd_rn(d, __fmul_rn(diff, diff));
+                        }
+                        const bool take = (c == 0) || (__fsub_rn(best, d) > 1e-6f);
+                        best = take ? d : best;
+                        bi = take ? c : bi;
+                    }
+                }
+                const uint32_t sh = 16 * (tg % 2) + 8 * pl + 4 * h;
+                uint32_t w = words[0];
+#pragma unroll
+                for (int i = 1; i < TG / 2; ++i) w = (tg / 2 == i) ? words[i] : w;
+                w = (w & ~(15u << sh)) | (bi << sh);
+#pragma unroll
+                for (int i = 0; i < TG / 2; ++i) words[i] = (tg / 2 == i) ? w : words[i];
+            }
+        }
+
+        // ---- merge the two codebooks of each pair (lanes l and l+32), gather the tile's index
+        //      bytes in LDS, store 8 bytes per token ------------------------------------------------
+#pragma unroll
+        for (int i = 0; i < TG / 2; ++i) words[i] |= __shfl_xor(words[i], 32);
+        if (h == 0) {
+#pragma unroll
+            for (int tg = 0; tg < TG; ++tg)
+                *reinterpret_cast<uint16_t*>(&ist[(32 * tg + j) * (CBW / 2) + 2 * wave]) =
+                    (uint16_t)(words[tg / 2] >> (16 * (tg % 2)));
+        }
+        __syncthreads();  // index bytes complete; every wave is done with the activation tile
+        if (threadIdx.x < TT) {
+            const uint32_t tok = tok0 + threadIdx.x;
+            if (tok < N) {
+                const uint2 w = *reinterpret_cast<const uint2*>(&ist[threadIdx.x * (CBW / 2)]);
+                if (idx_tiled) {
+                    *reinterpret_cast<uint32_t*>(idx + idx_offset(tok, tcb * (CBW / 2), idx_row_bytes, 1)) = w.x;
+                    *reinterpret_cast<uint32_t*>(idx + idx_offset(tok, tcb * (CBW / 2) + 4, idx_row_bytes, 1)) = w.y;
+                } else {
+                    *reinterpret_cast<uint2*>(idx + (size_t)tok * idx_row_bytes + tcb * (CBW / 2)) = w;
+                }
+            }
+        }
+    }
+}
+
 // Generic sub-vector length (any v): one lane per (token, codebook), operands straight from
 // global memory.  Correct for every shape; only used where no specialisation exists.
 template <int IDX_BITS>
@@ -734,10 +1048,47 @@ int launch_ccs_mfma(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d
     return hip_check(ctx, hipGetLastError(), "ccs_mfma_kernel launch");
 }
 
+// PIMDL_CCS_F32=1 keeps the fp32 matrix-core search for v = 4 (same results; for comparison)
+static bool ccs_f32_only()
+{
+    static const bool v = [] {
+        const char* e = getenv("PIMDL_CCS_F32");
+        return e && e[0] == '1';
+    }();
+    return v;
+}
+
+static int launch_ccs_bf16(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_cent, uint8_t* d_idx, uint32_t n)
+{
+    using S = CcsMfmaShape<4>;
+    const uint32_t tiles_cb = g.CB_pad / S::CBW;  // CB_pad is a multiple of 32
+    const uint64_t total64 = (uint64_t)((n + S::TILE_TOKENS - 1) / S::TILE_TOKENS) * tiles_cb;
+    if (total64 > 0xFFFFFFFFull) return set_error(ctx, PIMDL_ERR_INVALID, "ccs: too many tiles");
+    const uint32_t total = (uint32_t)total64;
+    int per_cu = 0;  // persistent grid: exactly the workgroups that are resident at once
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, ccs_bf16_kernel, CCS_THREADS, 0) != hipSuccess || per_cu < 1) {
+        (void)hipGetLastError();
+        per_cu = 1;
+    }
+    const uint32_t slots = (uint32_t)ctx->prop.multiProcessorCount * (uint32_t)per_cu;
+    dim3 grid(total < slots ? total : slots);
+    const int vec_ok = (g.K % 4 == 0) && ((reinterpret_cast<uintptr_t>(d_x) & 15) == 0);
+    const float* aux = d_cent + (size_t)g.CB * g.C * g.v;
+    const float* cnmax = aux + ccs_aux_floats(g);
+    const float* cnmax_pad = cnmax + g.CB + (size_t)(g.CB_pad / 2) * (g.v + 1) * 64;
+    const float* bf = d_cent + ccs_bf16_offset(g);
+    const uint4* aux_b = reinterpret_cast<const uint4*>(bf);
+    const float* cn16 = bf + (size_t)(g.CB_pad / 2) * 3 * 64 * 4;
+    hipLaunchKernelGGL(ccs_bf16_kernel, grid, dim3(CCS_THREADS), 0, ctx->stream, d_x, d_cent, aux_b, cn16, cnmax_pad,
+                       d_idx, n, g.K, g.CB, g.C, g.idx_row_bytes, (int)g.idx_tiled, vec_ok, tiles_cb, total);
+    return hip_check(ctx, hipGetLastError(), "ccs_bf16_kernel launch");
+}
+
 template <int IDX_BITS>
 int launch_ccs_bits(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_cent, uint8_t* d_idx, uint32_t n)
 {
     if (IDX_BITS == 4 && !ccs_exact_only()) {
+        if (g.v == 4 && !ccs_f32_only()) return launch_ccs_bf16(ctx, g, d_x, d_cent, d_idx, n);
         switch (g.v) {
             case 2: return launch_ccs_mfma<2>(ctx, g, d_x, d_cent, d_idx, n);
             case 4: return launch_ccs_mfma<4>(ctx, g, d_x, d_cent, d_idx, n);
@@ -776,7 +1127,7 @@ bool ccs_exact_only()
 
 size_t ccs_centroid_bytes(const AmmGeom& g)
 {
-    return ((size_t)g.CB * g.C * g.v + ccs_aux_floats(g) + g.CB + ccs_aux_a_floats(g)) * sizeof(float);
+    return (ccs_bf16_offset(g) + ccs_bf16_floats(g)) * sizeof(float);
 }
 
 int launch_ccs_prep(Ctx* ctx, const AmmGeom& g, float* d_cent)
@@ -790,7 +1141,12 @@ int launch_ccs_prep(Ctx* ctx, const AmmGeom& g, float* d_cent)
     float* aux_a = cnmax + g.CB;
     hipLaunchKernelGGL(ccs_prep_mfma_kernel, dim3(g.CB_pad / 2), dim3(64), 0, ctx->stream, d_cent, cnmax, aux_a,
                        aux_a + (size_t)(g.CB_pad / 2) * (g.v + 1) * 64, g.CB, g.C, g.v);
-    return hip_check(ctx, hipGetLastError(), "ccs_prep_mfma_kernel launch");
+    rc = hip_check(ctx, hipGetLastError(), "ccs_prep_mfma_kernel launch");
+    if (rc || !ccs_has_bf16(g)) return rc;
+    float* bf = d_cent + ccs_bf16_offset(g);
+    hipLaunchKernelGGL(ccs_prep_bf16_kernel, dim3(g.CB_pad / 2), dim3(64), 0, ctx->stream, d_cent,
+                       reinterpret_cast<uint4*>(bf), bf + (size_t)(g.CB_pad / 2) * 3 * 64 * 4, g.CB, g.C);
+    return hip_check(ctx, hipGetLastError(), "ccs_prep_bf16_kernel launch");
 }
 
 uint32_t ccs_cb_per_wg(uint32_t v)
