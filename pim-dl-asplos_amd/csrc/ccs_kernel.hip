@@ -683,7 +683,7 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
                                                                  uint8_t* __restrict__ idx, uint32_t N,
                                                                  uint32_t K, uint32_t CB, uint32_t C,
                                                                  uint32_t idx_row_bytes, int idx_tiled, int vec_ok,
-                                                                 uint32_t tiles_cb, uint32_t total_tiles)
+                                                                 uint32_t tiles_cb, uint32_t total_tiles, uint32_t num_cus)
 {
     constexpr int V = 4;
     using S = CcsMfmaShape<V>;
@@ -727,7 +727,20 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
     float4 pf[PASSES];
     if (blockIdx.x < total_tiles) fetch(pf, blockIdx.x);
 
+    // The CU issues from its oldest waves first, so of the workgroups resident on a CU the first one
+    // placed would finish its (equal) share of tiles well before the last and leave the CU half empty.
+    // A wave's priority falls as its workgroup progresses through its share: whoever is behind goes first.
+    const uint32_t my_tiles = (total_tiles - blockIdx.x + gridDim.x - 1) / gridDim.x;
+    uint32_t tiles_done = 0;
+    (void)num_cus;
     for (uint32_t tile_id = blockIdx.x; tile_id < total_tiles; tile_id += gridDim.x) {
+        switch (4 * tiles_done / my_tiles) {
+            case 0: __builtin_amdgcn_s_setprio(3); break;
+            case 1: __builtin_amdgcn_s_setprio(2); break;
+            case 2: __builtin_amdgcn_s_setprio(1); break;
+            default: __builtin_amdgcn_s_setprio(0); break;
+        }
+        ++tiles_done;
         const uint32_t tok0 = (tile_id / tiles_cb) * TT;
         const uint32_t tcb = tile_id % tiles_cb;          // codebooks 16 tcb .. 16 tcb + 15
         const uint32_t pair0 = tcb * (CBW / 2) + 2 * wave;  // first of this wave's two pairs
@@ -1080,7 +1093,8 @@ static int launch_ccs_bf16(Ctx* ctx, const AmmGeom& g, const float* d_x, const f
     const uint4* aux_b = reinterpret_cast<const uint4*>(bf);
     const float* cn16 = bf + (size_t)(g.CB_pad / 2) * 3 * 64 * 4;
     hipLaunchKernelGGL(ccs_bf16_kernel, grid, dim3(CCS_THREADS), 0, ctx->stream, d_x, d_cent, aux_b, cn16, cnmax_pad,
-                       d_idx, n, g.K, g.CB, g.C, g.idx_row_bytes, (int)g.idx_tiled, vec_ok, tiles_cb, total);
+                       d_idx, n, g.K, g.CB, g.C, g.idx_row_bytes, (int)g.idx_tiled, vec_ok, tiles_cb, total,
+                       (uint32_t)ctx->prop.multiProcessorCount);
     return hip_check(ctx, hipGetLastError(), "ccs_bf16_kernel launch");
 }
 
