@@ -72,8 +72,20 @@ def model_forward(pimdl, ctx, iters=10):
         model.forward(x)
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) * 1e3 / iters
+    # the same forward recorded once into a HIP graph and replayed (no host work between the kernels)
+    graph, _sx, _sy = model.capture(x)
+    for _ in range(3):
+        graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        graph.replay()
+    torch.cuda.synchronize()
+    ms_graph = (time.perf_counter() - t0) * 1e3 / iters
+    del graph
     model.close()
     return {"layers": 12, "tokens": p.n, "ms_per_forward": ms, "tokens_per_s": p.n / (ms * 1e-3),
+            "ms_per_forward_graph": ms_graph, "tokens_per_s_graph": p.n / (ms_graph * 1e-3),
             "note": "LUT-AMM linears + pimdl_layer_norm on libpimdl, attention and tanh-GELU in PyTorch-ROCm fp32"}
 
 

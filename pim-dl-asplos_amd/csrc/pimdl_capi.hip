@@ -619,7 +619,7 @@ int pimdl_layer_norm(pimdl_ctx* ctx, const float* x, const float* weight, const 
     const size_t row_bytes = (size_t)d * sizeof(float), mat_bytes = (size_t)n * row_bytes;
     struct Tmp {
         void* p = nullptr;
-        ~Tmp() { (void)hipFree(p); }
+        ~Tmp() { if (p) (void)hipFree(p); }
     } tx, tw, tb, tr, to;
     auto to_dev = [&](const float* h, size_t bytes, Tmp& t, const float** dptr) -> int {
         if (is_device_ptr(h)) {

@@ -240,6 +240,31 @@ class Transformer:
             x = layer.forward(x)
         return x
 
+    def capture(self, x):
+        """Records one forward pass on `x`'s shape into a HIP graph and returns (graph, static_input,
+        static_output): copy new features into static_input, graph.replay(), read static_output.
+        A layer is ~30 short kernels; launched one by one from Python the GPU waits for the host
+        about a third of the time, replayed from a graph it does not.  The library's calls are
+        recorded like any other launch (they run on the stream the context is bound to and, for
+        device buffers that have been seen before, allocate and synchronise nothing)."""
+        torch = self.layers[0].torch
+        ctx = self.layers[0].ctx
+        side = torch.cuda.Stream()
+        static_x = x.clone()
+        side.wait_stream(torch.cuda.current_stream())
+        ctx.set_stream(side.cuda_stream)
+        try:
+            with torch.cuda.stream(side):
+                for _ in range(2):  # first calls size the context's scratch and set kernel attributes
+                    self.forward(static_x)
+            side.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side, capture_error_mode="thread_local"):
+                static_y = self.forward(static_x)
+        finally:
+            ctx.set_stream(torch.cuda.current_stream().cuda_stream)
+        return graph, static_x, static_y
+
 
 def synth_layers(params, ctx, pimdl, seed=0, shared_qkv_centroids=False):
     """Random-init weights of the right shapes (what the reference's driver falls back to without a

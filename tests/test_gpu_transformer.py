@@ -139,6 +139,29 @@ def test_model_is_the_chain_of_its_layers_and_reads_the_weight_file(ctx, tmp_pat
     model.close()
 
 
+def test_captured_forward_replays_like_the_eager_one(ctx):
+    """The model forward recorded into a HIP graph: every replay, with eager work and synchronisations
+    in between and with new input copied into the static buffer, equals the eager result bit for bit."""
+    import torch
+    p = T.TransformerParams.from_yaml(CFG)
+    model = T.Transformer(ctx, pimdl, T.synth_layers(p, ctx, pimdl, seed=9), p)
+    gen = torch.Generator(device="cuda").manual_seed(4)
+    xs = [torch.randn((p.n, p.token_dim), device="cuda", generator=gen) for _ in range(3)]
+    want = [model.forward(x).clone() for x in xs]
+    torch.cuda.synchronize()
+    graph, static_x, static_y = model.capture(xs[0])
+    for rep in range(2):
+        for x, w in zip(xs, want):
+            static_x.copy_(x)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(static_y, w)
+            assert torch.equal(model.forward(xs[1]), want[1])  # eager work between replays, same context
+            torch.cuda.synchronize()
+    del graph
+    model.close()
+
+
 def test_driver_prints_the_reference_wording(capsys):
     assert T.main([CFG, "--iters", "2"]) == 0
     out = capsys.readouterr().out
