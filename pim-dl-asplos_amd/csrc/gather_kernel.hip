@@ -431,8 +431,9 @@ __global__ __launch_bounds__(GATHER_THREADS, 4) void gather_i8_kernel(
 // =============================================================================================
 constexpr int OH_WAVES = 4;
 constexpr int OH_THREADS = OH_WAVES * 64;
-constexpr int OH_TM = 4;                              // 16-token groups per wave
-constexpr int OH_TOK_ITEM = OH_WAVES * OH_TM * 16;    // 256 tokens per item
+// 16-token groups per wave (TM): 4 (256-token items) where the batch offers enough items to put two
+// workgroups on every CU, else 2 (128-token items, twice as many of them)
+constexpr int oh_tok_item(int tm) { return OH_WAVES * tm * 16; }
 
 // codebooks per slice (4 per MFMA K-step)
 constexpr int oh_slice_cbs(int) { return 16; }
@@ -441,7 +442,8 @@ constexpr int oh_nbuf(int) { return 3; }
 // one-hot table + LUT slice buffers + index buffers
 constexpr int oh_lds_bytes(int tn)
 {
-    return 256 + oh_nbuf(tn) * oh_slice_cbs(tn) * 16 * tn * 16 + oh_nbuf(tn) * OH_TOK_ITEM * (oh_slice_cbs(tn) / 2);
+    // (every wave keeps the index words of a whole 64-token block, whatever part of it it owns)
+    return 256 + oh_nbuf(tn) * oh_slice_cbs(tn) * 16 * tn * 16 + oh_nbuf(tn) * OH_WAVES * 64 * (oh_slice_cbs(tn) / 2);
 }
 
 // Loads through the scalar data cache (read only) of wave-uniform addresses; they count on the
@@ -460,20 +462,16 @@ __device__ __forceinline__ float scalar_load1(const float* p)
     return r;
 }
 
-// all operands of one K-step have landed; the registers pass through the asm so that no consumer
-// can be scheduled ahead of the wait
-template <int TN>
-__device__ __forceinline__ void oh_wait(v4i (&a)[TN], v4i (&b)[OH_TM])
+// all operands of one K-step have landed; the registers pass through (empty, ordered) asm statements
+// so that no consumer can be scheduled ahead of the wait
+template <int TN, int TM>
+__device__ __forceinline__ void oh_wait(v4i (&a)[TN], v4i (&b)[TM])
 {
-    static_assert(OH_TM == 4, "operand list");
-    if constexpr (TN == 3)
-        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
-    else if constexpr (TN == 4)
-        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
-    else {
-        static_assert(TN == 6, "operand list");
-        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
-    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < TN; ++i) asm volatile("" : "+v"(a[i]));
+#pragma unroll
+    for (int i = 0; i < TM; ++i) asm volatile("" : "+v"(b[i]));
 }
 
 // A workgroup is four waves; wave w owns tokens 64 w .. 64 w + 63 of a 256-token tile (TM = 4) and
@@ -481,13 +479,14 @@ __device__ __forceinline__ void oh_wait(v4i (&a)[TN], v4i (&b)[OH_TM])
 // can only issue an MFMA every ~30 cycles; two keep the matrix core at its ~21).  Smaller wave
 // tiles with more waves were slower: a K-step must hold enough MFMAs (TM*TN) to cover the LDS
 // latency of the next K-step's operands.
-template <int TN>
+template <int TN, int TM>
 __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
     const uint8_t* __restrict__ idx, const int8_t* __restrict__ lut, float* __restrict__ out,
     int32_t* __restrict__ acc_out, uint32_t N, uint32_t M, uint32_t CB_pad, uint32_t idx_row_bytes,
     uint32_t n_token_tiles, uint32_t n_items, Epilogue ep)
 {
-    constexpr int TM = OH_TM;
+    constexpr int OH_TOK_ITEM = oh_tok_item(TM);
+    static_assert(TM == 4 || TM == 2, "a wave owns a whole or half a 64-token index block");
     constexpr int WN = 16 * TN;                    // columns per item
     constexpr int G = oh_slice_cbs(TN);            // codebooks per slice
     constexpr int SLICE = G * WN * 16;             // bytes of one codebook slice
@@ -503,7 +502,7 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
     constexpr int PD = NBUF - 1;  // prefetch distance of the LUT stream, in slices
     constexpr uint32_t BUF0 = 256;  // the table sits at LDS offset 0: entry address = nibble * 16
     constexpr uint32_t IBUF0 = BUF0 + NBUF * SLICE;
-    constexpr uint32_t IBYTES = OH_TOK_ITEM * (G / 2);        // index bytes of one slice
+    constexpr uint32_t IBYTES = OH_WAVES * 64 * (G / 2);      // index bytes of one slice (a 64-token block per wave)
     constexpr uint32_t IWAVE = 64 * (G / 2);                  // ... of one wave's 64 tokens
     constexpr int IX_OPS = IWORDS;                            // 64 lanes x 4 B = 64 tokens x 1 word
     constexpr int DMA_OPS = DMA_PER_WAVE + IX_OPS;            // memory operations per wave and slice
@@ -545,7 +544,8 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
     // is one contiguous 256-byte block (see idx_offset).
     const uint32_t last_block = (N - 1) / 64;
     auto locate_ix = [&]() {
-        uint32_t blk = (ix_item % n_token_tiles) * (OH_TOK_ITEM / 64) + wave;
+        // TM = 4: wave w owns block w of the tile; TM = 2: waves 2p and 2p+1 each copy block p and own half of it
+        uint32_t blk = ((ix_item % n_token_tiles) * OH_TOK_ITEM + wave * (TM * 16)) / 64;
         if (blk > last_block) blk = last_block;  // clamp: results of such tokens are never stored
         ix_base = idx + (size_t)blk * idx_row_bytes * 64;
         ix_lane_off = lane * 4;
@@ -598,7 +598,7 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
     // after masking, one v_bfe_u32 yields nibble * 16: the byte offset of the one-hot table entry.
     const uint32_t pre_shift = (g & 1) ? 0u : 4u;
     const uint32_t byte_shift = 8 * (g >> 1);
-    const uint32_t ix_lane = IBUF0 + wave * IWAVE + j * 4;
+    const uint32_t ix_lane = IBUF0 + wave * IWAVE + (((wave * (TM * 16)) & 63) + j) * 4;
     // The index words are read with inline assembly: the compiler cannot tell these reads from the
     // LDS ranges the copy operations in flight are writing, and would wait for all of them first.
     auto read_ix = [&](uint32_t (&raw)[TM][IWORDS], uint32_t ibuf) {
@@ -609,17 +609,11 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
         });
     };
     auto unpack_ix = [&](uint32_t (&iwm)[TM][IWORDS], uint32_t (&raw)[TM][IWORDS]) {
-        static_assert(TM == 4 && (IWORDS == 2 || IWORDS == 4), "operand list of the wait");
-        if constexpr (IWORDS == 2)
-            asm volatile("s_waitcnt lgkmcnt(0)"
-                         : "+v"(raw[0][0]), "+v"(raw[0][1]), "+v"(raw[1][0]), "+v"(raw[1][1]), "+v"(raw[2][0]),
-                           "+v"(raw[2][1]), "+v"(raw[3][0]), "+v"(raw[3][1]));
-        else
-            asm volatile("s_waitcnt lgkmcnt(0)"
-                         : "+v"(raw[0][0]), "+v"(raw[0][1]), "+v"(raw[0][2 % IWORDS]), "+v"(raw[0][3 % IWORDS]),
-                           "+v"(raw[1][0]), "+v"(raw[1][1]), "+v"(raw[1][2 % IWORDS]), "+v"(raw[1][3 % IWORDS]),
-                           "+v"(raw[2][0]), "+v"(raw[2][1]), "+v"(raw[2][2 % IWORDS]), "+v"(raw[2][3 % IWORDS]),
-                           "+v"(raw[3][0]), "+v"(raw[3][1]), "+v"(raw[3][2 % IWORDS]), "+v"(raw[3][3 % IWORDS]));
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int t = 0; t < TM; ++t)
+#pragma unroll
+            for (int i = 0; i < IWORDS; ++i) asm volatile("" : "+v"(raw[t][i]));
 #pragma unroll
         for (int t = 0; t < TM; ++t)
 #pragma unroll
@@ -769,7 +763,7 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
         issue_reads(std::integral_constant<int, 0>{});
         static_for<0, KSTEPS>([&](auto ksc) {
             constexpr int ks = decltype(ksc)::value;
-            oh_wait<TN>(a_op[ks & 1], b_op[ks & 1]);
+            oh_wait<TN, TM>(a_op[ks & 1], b_op[ks & 1]);
             if constexpr (ks + 1 < KSTEPS) issue_reads(std::integral_constant<int, ks + 1>{});
             // the next slice's index words (this wave's own copy, landed before the wait above)
             if constexpr (ks == KSTEPS - 1) read_ix(iw_raw, ibuf_next);
@@ -799,12 +793,13 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
     }
 }
 
-template <int TN>
-int launch_onehot(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_t* d_acc, uint32_t n,
-                  const Epilogue& ep)
+template <int TN, int TM>
+int launch_onehot_tm(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_t* d_acc, uint32_t n,
+                     const Epilogue& ep)
 {
     constexpr int LDS = oh_lds_bytes(TN);
-    auto kern = gather_onehot_kernel<TN>;
+    constexpr int OH_TOK_ITEM = oh_tok_item(TM);
+    auto kern = gather_onehot_kernel<TN, TM>;
     static bool attr_set = false;
     if (!attr_set) {
         int rc = hip_check(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -821,6 +816,17 @@ int launch_onehot(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, in
                        reinterpret_cast<const int8_t*>(a.d_lut), d_out, d_acc, n, a.g.M, a.g.CB_pad,
                        a.g.idx_row_bytes, n_token_tiles, n_items, ep);
     return hip_check(ctx, hipGetLastError(), "gather_onehot_kernel launch");
+}
+
+// 256-token items (TM = 4) need fewer LDS reads and copies per MFMA; when the batch does not offer
+// two of them per CU, 128-token items (TM = 2) put a second wave on every SIMD instead.
+template <int TN>
+int launch_onehot(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_t* d_acc, uint32_t n,
+                  const Epilogue& ep)
+{
+    const uint64_t items4 = (uint64_t)((n + oh_tok_item(4) - 1) / oh_tok_item(4)) * (a.g.M_pad / (16 * TN));
+    if (items4 < 2ull * ctx->prop.multiProcessorCount) return launch_onehot_tm<TN, 2>(ctx, a, d_idx, d_out, d_acc, n, ep);
+    return launch_onehot_tm<TN, 4>(ctx, a, d_idx, d_out, d_acc, n, ep);
 }
 
 // ---------------------------------------------------------------------------------------------
