@@ -210,8 +210,10 @@ class TransformerLayer:
         else:
             q, k, v = self._run("q", x, n), self._run("k", x, n), self._run("v", x, n)
         qh, kh, vh = (t.reshape(B, S, H, hd).permute(0, 2, 1, 3) for t in (q, k, v))
-        scores = torch.matmul(qh, kh.transpose(-1, -2)) * (1.0 / math.sqrt(p.token_dim / p.head_num))
-        attn = torch.matmul(torch.softmax(scores, dim=-1), vh)               # [B][H][S][hd]
+        # unmasked softmax(q k^T / sqrt(head_dim)) v in fp32; the fused kernel reads the strided head views
+        # directly (separate matmul / softmax calls first copy each of them into [B][H][S][hd] order)
+        attn = torch.nn.functional.scaled_dot_product_attention(
+            qh, kh, vh, scale=1.0 / math.sqrt(p.token_dim / p.head_num))     # [B][H][S][hd]
         a = attn.permute(0, 2, 1, 3).reshape(n, p.token_dim).contiguous()
         o = self._run("o", a, n)
         h = self._norm_residual("attention_norm", o, x)
