@@ -150,10 +150,14 @@ def load_npz(path, params):
 class TransformerLayer:
     """One encoder layer resident on the GPU: six LUT-AMM operators and two LayerNorms."""
 
-    def __init__(self, ctx, pimdl, weights, params, fused_qkv=False):
+    def __init__(self, ctx, pimdl, weights, params, fused_qkv=False, side=None):
+        """side: optional ((context, torch stream), (context, torch stream)) for the K and V projections.
+        The three projections read the same input and are independent; at small batches each of them
+        fills only half of the GPU, so running them on three streams overlaps them."""
         import torch
         self.ctx, self.params, self.torch = ctx, params, torch
         self.fused_qkv = fused_qkv
+        self.side = None if fused_qkv else side
         n = params.n
         self.amm = {}
         lin = dict(weights)
@@ -169,8 +173,11 @@ class TransformerLayer:
         for name in names:
             w = lin[name]
             # bias_mode: pim_lut's epilogue adds lut_bias * num_codebook (pim_lut_host.cpp:201)
-            self.amm[name] = ctx.amm(w["centroids"], w["lut"], np.float32(w["scale"]), w["bias"], max_n=n,
-                                     lut_bias=float(w.get("lut_bias", 0.0)), bias_mode=pimdl.BIAS_TIMES_CB)
+            owner = ctx
+            if self.side and name in ("k", "v"):
+                owner = self.side[0 if name == "k" else 1][0]
+            self.amm[name] = owner.amm(w["centroids"], w["lut"], np.float32(w["scale"]), w["bias"], max_n=n,
+                                       lut_bias=float(w.get("lut_bias", 0.0)), bias_mode=pimdl.BIAS_TIMES_CB)
         dev = torch.device("cuda", torch.cuda.current_device())
         self.norm = {name: (torch.from_numpy(np.ascontiguousarray(weights[name]["weight"], np.float32)).to(dev),
                             torch.from_numpy(np.ascontiguousarray(weights[name]["bias"], np.float32)).to(dev))
@@ -207,6 +214,15 @@ class TransformerLayer:
         if self.fused_qkv:
             qkv = self._run("qkv", x, n)
             q, k, v = (qkv[:, i * p.token_dim:(i + 1) * p.token_dim] for i in range(3))
+        elif self.side:
+            main = torch.cuda.current_stream()
+            q, k, v = (torch.empty((n, p.token_dim), device=x.device, dtype=torch.float32) for _ in range(3))
+            for (_, stream), name, dst in zip(self.side, ("k", "v"), (k, v)):
+                stream.wait_stream(main)                                   # fork: x is ready
+                self.amm[name].run_ptr(x.data_ptr(), n, dst.data_ptr())    # queued on that context's stream
+            self.amm["q"].run_ptr(x.data_ptr(), n, q.data_ptr())
+            for _, stream in self.side:
+                main.wait_stream(stream)                                   # join
         else:
             q, k, v = self._run("q", x, n), self._run("k", x, n), self._run("v", x, n)
         qh, kh, vh = (t.reshape(B, S, H, hd).permute(0, 2, 1, 3) for t in (q, k, v))
@@ -229,13 +245,24 @@ class TransformerLayer:
 class Transformer:
     """layer_num encoder layers (transformer_model.cpp:13-49: each layer's output is the next one's input)."""
 
-    def __init__(self, ctx, pimdl, layers, params, fused_qkv=False):
-        self.layers = [TransformerLayer(ctx, pimdl, w, params, fused_qkv) for w in layers]
+    def __init__(self, ctx, pimdl, layers, params, fused_qkv=False, parallel_qkv=True):
+        import torch
+        self.side = None
+        if parallel_qkv and not fused_qkv:
+            self.side = []
+            for _ in range(2):
+                c, st = pimdl.Context(torch.cuda.current_device()), torch.cuda.Stream()
+                c.set_stream(st.cuda_stream)
+                self.side.append((c, st))
+        self.layers = [TransformerLayer(ctx, pimdl, w, params, fused_qkv, self.side) for w in layers]
         self.params = params
 
     def close(self):
         for layer in self.layers:
             layer.close()
+        for c, _ in self.side or []:
+            c.close()
+        self.side = None
 
     def forward(self, x):
         for layer in self.layers:
