@@ -71,7 +71,9 @@ inline size_t ccs_aux_a_floats(const AmmGeom& g)
 
 // bf16-split search (v = 4, C <= 16): offset in floats of its operands behind everything else, and
 // their size.  The offset is rounded up to 16 bytes (uint4 operand images).
-inline bool ccs_has_bf16(const AmmGeom& g) { return g.v == 4 && g.C <= 16; }
+inline bool ccs_has_bf16(const AmmGeom& g) { return (g.v == 2 || g.v == 4 || g.v == 8) && g.C <= 16; }
+// MFMAs (16 K-slots each) per codebook pair: 2 codebooks x v dims x 6 cross products
+constexpr uint32_t ccs_bf16_nm(uint32_t v) { return (12 * v + 15) / 16; }
 inline size_t ccs_bf16_offset(const AmmGeom& g)
 {
     const size_t o = (size_t)g.CB * g.C * g.v + ccs_aux_floats(g) + g.CB + ccs_aux_a_floats(g);
@@ -79,7 +81,7 @@ inline size_t ccs_bf16_offset(const AmmGeom& g)
 }
 inline size_t ccs_bf16_floats(const AmmGeom& g)
 {
-    return ccs_has_bf16(g) ? (size_t)(g.CB_pad / 2) * 3 * 64 * 4 + (size_t)g.CB_pad * 16 : 0;
+    return ccs_has_bf16(g) ? (size_t)(g.CB_pad / 2) * ccs_bf16_nm(g.v) * 64 * 4 + (size_t)g.CB_pad * 16 : 0;
 }
 
 template <int N, typename F>
@@ -614,60 +616,71 @@ __global__ __launch_bounds__(CCS_THREADS, 4) void ccs_mfma_kernel(const float* _
 }
 
 // =============================================================================================
-// bf16-split variant of the MFMA search for v = 4 (C <= 16).  The fp32 MFMA above shares the fp32
+// bf16-split variant of the MFMA search for v in {2, 4, 8} (C <= 16).  The fp32 MFMA above shares the fp32
 // units with the VALU, so its five instructions per item (147 ns) add to the ~50 VALU operations of
 // the top-two search (100 ns).  v_mfma_f32_32x32x16_bf16 is twice as fast per K-slot and runs beside
 // VALU work.  bf16 has 8 significand bits, so each fp32 value is cut into three bf16 pieces and six
 // of the nine cross products are kept (see `scores` below); the score then carries a known error
 // bound like the fp32 form's, only larger (A2 below), and everything after the scores -- tagged
 // keys, tournament, margin test, exact replay -- is the same.  Operands:
-//   aux_b [CB_pad/2 pairs][3][64 lanes] uint4  A-operand images (bf16 pieces of -2c, by K-slot)
+//   aux_b [CB_pad/2 pairs][NM][64 lanes] uint4 A-operand images (bf16 pieces of -2c, by K-slot)
 //   cn16  [CB_pad][16] float                   |c|^2 (r for padded codebooks, 3e38 for ids past C)
 // =============================================================================================
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
-// K-slot register rho (0..11, four per MFMA) of lane (row i, half kh) pairs dims 2kh, 2kh+1 of codebook
-// rho / 6 of the pair with piece  {ch, cm, ch, cm, cl, ch}[rho % 6]  of -2c; the search kernel supplies
-// {xh, xh, xm, xm, xh, xl} in the same registers.  Rows of the other codebook hold zeros there.
+// K-slot registers (two bf16 K-slots each, four registers per MFMA) of lane (row i, half kh).  The lane
+// covers dims DL*kh .. DL*kh + DL-1 (DL = v/2) of both codebooks of the pair; codebook q of the pair owns
+// registers 3*DL*q .. 3*DL*q + 3*DL-1:
+//   DL >= 2: six registers per pair of dims (d, d+1), each (piece of d | piece of d+1 << 16), pieces
+//            {ch, cm, ch, cm, cl, ch} of -2c against the search kernel's {xh, xh, xm, xm, xh, xl};
+//   DL == 1: three registers for the one dim, (ch | cm), (ch | cm), (cl | ch) against (xh | xh), (xm | xm), (xh | xl).
+// Rows of the other codebook, and registers past 6*DL, hold zeros.
+template <uint32_t V>
 __global__ void ccs_prep_bf16_kernel(const float* __restrict__ cent, uint4* __restrict__ aux_b,
                                      float* __restrict__ cn16, uint32_t CB, uint32_t C)
 {
-    constexpr uint32_t v = 4;
+    constexpr uint32_t DL = V / 2, NM = ccs_bf16_nm(V);
     const uint32_t pair = blockIdx.x, lane = threadIdx.x;
     const uint32_t i = lane & 31, kh = lane >> 5;
     const uint32_t h = (i >> 2) & 1, r = (i & 3) + 4 * (i >> 3);
     const uint32_t cb = 2 * pair + h;
     const bool real = (cb < CB) && (r < C);
-    const float* cp = cent + ((size_t)cb * C + r) * v;
-    uint32_t piece[3] = {0, 0, 0};  // (dim 2kh | dim 2kh+1 << 16) of ch, cm, cl
-    if (real) {
-        uint32_t pc[2][3];
-        for (int d = 0; d < 2; ++d) {
-            const float a = -2.0f * cp[2 * kh + d];
-            const uint32_t au = __float_as_uint(a);
-            const float r1 = __fsub_rn(a, __uint_as_float(au & 0xffff0000u));
-            const uint32_t r1u = __float_as_uint(r1);
-            const float r2 = __fsub_rn(r1, __uint_as_float(r1u & 0xffff0000u));
-            pc[d][0] = au >> 16;
-            pc[d][1] = r1u >> 16;
-            pc[d][2] = __float_as_uint(r2) >> 16;
-        }
-        for (int t = 0; t < 3; ++t) piece[t] = pc[0][t] | (pc[1][t] << 16);
+    const float* cp = cent + ((size_t)cb * C + r) * V;
+    uint32_t pc[DL][3];  // bf16 pieces ch, cm, cl of -2c for the lane's dims
+    for (uint32_t d = 0; d < DL; ++d) {
+        const float a = real ? -2.0f * cp[DL * kh + d] : 0.0f;
+        const uint32_t au = __float_as_uint(a);
+        const float r1 = __fsub_rn(a, __uint_as_float(au & 0xffff0000u));
+        const uint32_t r1u = __float_as_uint(r1);
+        const float r2 = __fsub_rn(r1, __uint_as_float(r1u & 0xffff0000u));
+        pc[d][0] = au >> 16;
+        pc[d][1] = r1u >> 16;
+        pc[d][2] = __float_as_uint(r2) >> 16;
     }
     const int term[6] = {0, 1, 0, 1, 2, 0};
-    for (uint32_t m = 0; m < 3; ++m) {
+    for (uint32_t m = 0; m < NM; ++m) {
         uint32_t w[4];
         for (uint32_t q = 0; q < 4; ++q) {
             const uint32_t rho = 4 * m + q;
-            w[q] = (rho / 6 == h) ? piece[term[rho % 6]] : 0u;
+            uint32_t val = 0;
+            if (real && rho < 6 * DL && rho / (3 * DL) == h) {
+                const uint32_t sg = rho % (3 * DL);
+                if (DL == 1) {
+                    val = sg == 2 ? (pc[0][2] | (pc[0][0] << 16)) : (pc[0][0] | (pc[0][1] << 16));
+                } else {
+                    const uint32_t dp = sg / 6, t = term[sg % 6];
+                    val = pc[2 * dp][t] | (pc[2 * dp + 1][t] << 16);
+                }
+            }
+            w[q] = val;
         }
-        aux_b[((size_t)pair * 3 + m) * 64 + lane] = make_uint4(w[0], w[1], w[2], w[3]);
+        aux_b[((size_t)pair * NM + m) * 64 + lane] = make_uint4(w[0], w[1], w[2], w[3]);
     }
     if (kh == 0) {
         float cn = (float)r;  // a padded codebook scores r against centroid r: index 0 with a margin of 1
         if (real) {
             cn = 0.0f;
-            for (uint32_t t = 0; t < v; ++t) cn = fmaf(cp[t], cp[t], cn);
+            for (uint32_t t = 0; t < V; ++t) cn = fmaf(cp[t], cp[t], cn);
         } else if (cb < CB) {
             cn = 3e38f;  // centroid ids past C never win
         }
@@ -675,6 +688,7 @@ __global__ void ccs_prep_bf16_kernel(const float* __restrict__ cent, uint4* __re
     }
 }
 
+template <int V>
 __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* __restrict__ x,
                                                                  const float* __restrict__ cent,
                                                                  const uint4* __restrict__ aux_b,
@@ -685,10 +699,10 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
                                                                  uint32_t idx_row_bytes, int idx_tiled, int vec_ok,
                                                                  uint32_t tiles_cb, uint32_t total_tiles, uint32_t num_cus)
 {
-    constexpr int V = 4;
     using S = CcsMfmaShape<V>;
     constexpr int TF = S::TF, PITCH = S::PITCH, TT = S::TILE_TOKENS, CBW = S::CBW, TG = S::TG;
-    constexpr int NM = 3;  // MFMAs per item: 2 codebooks x 4 dims x 6 cross terms = 48 K-slots
+    constexpr int NM = (int)ccs_bf16_nm(V);  // MFMAs per item: 2 codebooks x v dims x 6 cross products, 16 K-slots each
+    constexpr int DL = V / 2;                // dims of each codebook this lane supplies
     constexpr int ITEMS = S::ITEMS;
     __shared__ __attribute__((aligned(16))) float tile[S::X_FLOATS];
     __shared__ __attribute__((aligned(16))) float cst[S::CENT_FLOATS];
@@ -771,16 +785,33 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
         if (tile_id + gridDim.x < total_tiles) fetch(pf, tile_id + gridDim.x);
 
         // Scores of item `it` (pair pl, token group tg) for this lane's token: this lane (half h) holds
-        // dims 2h, 2h+1 of both codebooks of the pair.  Each value is cut into three bf16 pieces by
-        // masking (x = xh + xm + xl exactly: 8 + 8 + 8 significand bits); the A operand holds the same
+        // dims DL*h .. DL*h + DL-1 of both codebooks of the pair.  Each value is cut into three bf16 pieces
+        // by masking (x = xh + xm + xl exactly: 8 + 8 + 8 significand bits); the A operand holds the same
         // pieces of -2c, and the K-slots pair them as  xh*ch, xh*cm, xm*ch, xm*cm, xh*cl, xl*ch  (the three
         // omitted products are below 2^-20 |x||c|).  Products of bf16 values are exact in fp32; the
         // accumulators start from |c|^2.  xx_out: |x|^2 over the lane's own codebook (for the bound).
         auto scores = [&](floatx16& acc, float& xx_out, int it) {
             const int pl = it / TG, tg = it % TG;
             const float* brow = brow0 + tg * 32 * PITCH + pl * 2 * V;
-            const float2 x0 = *reinterpret_cast<const float2*>(brow + 2 * h);      // codebook 0 of the pair
-            const float2 x1 = *reinterpret_cast<const float2*>(brow + V + 2 * h);  // codebook 1
+            float xs[2][DL];
+#pragma unroll
+            for (int cbh = 0; cbh < 2; ++cbh) {
+                const float* src = brow + cbh * V + DL * h;
+                if constexpr (DL == 1) {
+                    xs[cbh][0] = src[0];
+                } else if constexpr (DL == 2) {
+                    const float2 t2 = *reinterpret_cast<const float2*>(src);
+                    xs[cbh][0] = t2.x;
+                    xs[cbh][1] = t2.y;
+                } else {
+                    static_assert(DL == 4, "dims per lane");
+                    const float4 t4 = *reinterpret_cast<const float4*>(src);
+                    xs[cbh][0] = t4.x;
+                    xs[cbh][1] = t4.y;
+                    xs[cbh][2] = t4.z;
+                    xs[cbh][3] = t4.w;
+                }
+            }
             const float4* cnp = reinterpret_cast<const float4*>(cnl + (2 * (2 * wave + pl) + h) * 16);
 #pragma unroll
             for (int q4 = 0; q4 < 4; ++q4) {
@@ -790,29 +821,53 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
                 acc[4 * q4 + 2] = c4.z;
                 acc[4 * q4 + 3] = c4.w;
             }
-            uint32_t H[2], Mm[2], L[2];
+            uint32_t breg[NM * 4];
+#pragma unroll
+            for (int i = 0; i < NM * 4; ++i) breg[i] = 0;
             float part[2];
 #pragma unroll
             for (int cbh = 0; cbh < 2; ++cbh) {
-                const float a = cbh ? x1.x : x0.x, b = cbh ? x1.y : x0.y;
-                const uint32_t au = __float_as_uint(a), bu = __float_as_uint(b);
-                const float ar1 = a - __uint_as_float(au & 0xffff0000u), br1 = b - __uint_as_float(bu & 0xffff0000u);
-                const uint32_t ar1u = __float_as_uint(ar1), br1u = __float_as_uint(br1);
-                const float ar2 = ar1 - __uint_as_float(ar1u & 0xffff0000u), br2 = br1 - __uint_as_float(br1u & 0xffff0000u);
-                H[cbh] = __builtin_amdgcn_perm(bu, au, 0x07060302u);       // (bf16 of dim 2h | bf16 of dim 2h+1 << 16)
-                Mm[cbh] = __builtin_amdgcn_perm(br1u, ar1u, 0x07060302u);
-                L[cbh] = __builtin_amdgcn_perm(__float_as_uint(br2), __float_as_uint(ar2), 0x07060302u);
-                part[cbh] = fmaf(b, b, a * a);
+                uint32_t xu[DL], r1u[DL], r2u[DL];
+                float sq = 0.0f;
+#pragma unroll
+                for (int d = 0; d < DL; ++d) {
+                    const float a = xs[cbh][d];
+                    xu[d] = __float_as_uint(a);
+                    const float r1 = a - __uint_as_float(xu[d] & 0xffff0000u);
+                    r1u[d] = __float_as_uint(r1);
+                    r2u[d] = __float_as_uint(r1 - __uint_as_float(r1u[d] & 0xffff0000u));
+                    sq = d == 0 ? a * a : fmaf(a, a, sq);
+                }
+                part[cbh] = sq;
+                // __builtin_amdgcn_perm(p, q, 0x07060302) = (bf16 of q | bf16 of p << 16)
+                if constexpr (DL == 1) {
+                    breg[3 * cbh + 0] = __builtin_amdgcn_perm(xu[0], xu[0], 0x07060302u);    // (xh | xh)
+                    breg[3 * cbh + 1] = __builtin_amdgcn_perm(r1u[0], r1u[0], 0x07060302u);  // (xm | xm)
+                    breg[3 * cbh + 2] = __builtin_amdgcn_perm(r2u[0], xu[0], 0x07060302u);   // (xh | xl)
+                } else {
+#pragma unroll
+                    for (int dp = 0; dp < DL / 2; ++dp) {
+                        const uint32_t H = __builtin_amdgcn_perm(xu[2 * dp + 1], xu[2 * dp], 0x07060302u);
+                        const uint32_t Mm = __builtin_amdgcn_perm(r1u[2 * dp + 1], r1u[2 * dp], 0x07060302u);
+                        const uint32_t L = __builtin_amdgcn_perm(r2u[2 * dp + 1], r2u[2 * dp], 0x07060302u);
+                        const int r0 = 3 * DL * cbh + 6 * dp;
+                        breg[r0 + 0] = H;
+                        breg[r0 + 1] = H;
+                        breg[r0 + 2] = Mm;
+                        breg[r0 + 3] = Mm;
+                        breg[r0 + 4] = H;
+                        breg[r0 + 5] = L;
+                    }
+                }
             }
             // |x|^2 of codebook h: lanes l and l+32 each hold half of it for both codebooks
             const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(part[0]), __float_as_uint(part[1]), false, false);
             xx_out = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
-            const uint4 b0 = make_uint4(H[0], H[0], Mm[0], Mm[0]);
-            const uint4 b1 = make_uint4(H[0], L[0], H[1], H[1]);
-            const uint4 b2 = make_uint4(Mm[1], Mm[1], H[1], L[1]);
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, aq[pl][0]), __builtin_bit_cast(bf16x8, b0), acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, aq[pl][1]), __builtin_bit_cast(bf16x8, b1), acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, aq[pl][2]), __builtin_bit_cast(bf16x8, b2), acc, 0, 0, 0);
+#pragma unroll
+            for (int m = 0; m < NM; ++m) {
+                const uint4 bm = make_uint4(breg[4 * m], breg[4 * m + 1], breg[4 * m + 2], breg[4 * m + 3]);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, aq[pl][m]), __builtin_bit_cast(bf16x8, bm), acc, 0, 0, 0);
+            }
         };
 
         // words[tg / 2], 16 bits per token group: nibble of (pair pl, half h) at bit 8 pl + 4 h
@@ -849,9 +904,10 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
             const float m2 = vmin3(vmin3(md[0], md[1], md[2]), vmin3(md[3], md[4], vmax(a1, b1)), vmin(a2, b2));
             const uint32_t bi = __float_as_uint(m1) & 15u;
             const float mag = xx + cmax[pl];
-            // 2 * [ (v+1)u (|c|^2) + 16u (omitted products) + 103u (51 additions, each within u of a partial
-            //       sum below 2.02 mag) + 2(v+2)u (the reference's own chain) ] = 2 * 136u
-            constexpr float A2 = 2.0f * 136.0f * 5.9604645e-8f;
+            // 2 * [ (v+1)u (|c|^2) + 16u (omitted products) + 2.02 (12v + NM) u (that many additions, each
+            //       within u of a partial sum below 2.02 mag) + 2(v+2)u (the reference's own chain) ]
+            //       = 2 * {80, 136, 251} u  for v = {2, 4, 8}
+            constexpr float A2 = 2.0f * ((V + 1) + 16.0f + 2.02f * (12 * V + NM) + 2 * (V + 2)) * 5.9604645e-8f;
             constexpr float B2 = 2.0f * 16.0f * 2.3841858e-7f;               // 2 * 2^(4-22)
             const float thr = fmaf(A2, mag, fmaf(B2, fabsf(m2), 1.001e-6f));
             // NaN anywhere makes a compare false, which counts as "not safe"
@@ -1061,7 +1117,7 @@ int launch_ccs_mfma(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d
     return hip_check(ctx, hipGetLastError(), "ccs_mfma_kernel launch");
 }
 
-// PIMDL_CCS_F32=1 keeps the fp32 matrix-core search for v = 4 (same results; for comparison)
+// PIMDL_CCS_F32=1 keeps the fp32 matrix-core search (same results; for comparison)
 static bool ccs_f32_only()
 {
     static const bool v = [] {
@@ -1071,15 +1127,16 @@ static bool ccs_f32_only()
     return v;
 }
 
-static int launch_ccs_bf16(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_cent, uint8_t* d_idx, uint32_t n)
+template <int V>
+int launch_ccs_bf16(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_cent, uint8_t* d_idx, uint32_t n)
 {
-    using S = CcsMfmaShape<4>;
+    using S = CcsMfmaShape<V>;
     const uint32_t tiles_cb = g.CB_pad / S::CBW;  // CB_pad is a multiple of 32
     const uint64_t total64 = (uint64_t)((n + S::TILE_TOKENS - 1) / S::TILE_TOKENS) * tiles_cb;
     if (total64 > 0xFFFFFFFFull) return set_error(ctx, PIMDL_ERR_INVALID, "ccs: too many tiles");
     const uint32_t total = (uint32_t)total64;
     int per_cu = 0;  // persistent grid: exactly the workgroups that are resident at once
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, ccs_bf16_kernel, CCS_THREADS, 0) != hipSuccess || per_cu < 1) {
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, ccs_bf16_kernel<V>, CCS_THREADS, 0) != hipSuccess || per_cu < 1) {
         (void)hipGetLastError();
         per_cu = 1;
     }
@@ -1091,8 +1148,8 @@ static int launch_ccs_bf16(Ctx* ctx, const AmmGeom& g, const float* d_x, const f
     const float* cnmax_pad = cnmax + g.CB + (size_t)(g.CB_pad / 2) * (g.v + 1) * 64;
     const float* bf = d_cent + ccs_bf16_offset(g);
     const uint4* aux_b = reinterpret_cast<const uint4*>(bf);
-    const float* cn16 = bf + (size_t)(g.CB_pad / 2) * 3 * 64 * 4;
-    hipLaunchKernelGGL(ccs_bf16_kernel, grid, dim3(CCS_THREADS), 0, ctx->stream, d_x, d_cent, aux_b, cn16, cnmax_pad,
+    const float* cn16 = bf + (size_t)(g.CB_pad / 2) * ccs_bf16_nm(V) * 64 * 4;
+    hipLaunchKernelGGL(ccs_bf16_kernel<V>, grid, dim3(CCS_THREADS), 0, ctx->stream, d_x, d_cent, aux_b, cn16, cnmax_pad,
                        d_idx, n, g.K, g.CB, g.C, g.idx_row_bytes, (int)g.idx_tiled, vec_ok, tiles_cb, total,
                        (uint32_t)ctx->prop.multiProcessorCount);
     return hip_check(ctx, hipGetLastError(), "ccs_bf16_kernel launch");
@@ -1102,7 +1159,14 @@ template <int IDX_BITS>
 int launch_ccs_bits(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_cent, uint8_t* d_idx, uint32_t n)
 {
     if (IDX_BITS == 4 && !ccs_exact_only()) {
-        if (g.v == 4 && !ccs_f32_only()) return launch_ccs_bf16(ctx, g, d_x, d_cent, d_idx, n);
+        if (!ccs_f32_only()) {
+            switch (g.v) {
+                case 2: return launch_ccs_bf16<2>(ctx, g, d_x, d_cent, d_idx, n);
+                case 4: return launch_ccs_bf16<4>(ctx, g, d_x, d_cent, d_idx, n);
+                case 8: return launch_ccs_bf16<8>(ctx, g, d_x, d_cent, d_idx, n);
+                default: break;
+            }
+        }
         switch (g.v) {
             case 2: return launch_ccs_mfma<2>(ctx, g, d_x, d_cent, d_idx, n);
             case 4: return launch_ccs_mfma<4>(ctx, g, d_x, d_cent, d_idx, n);
@@ -1158,8 +1222,14 @@ int launch_ccs_prep(Ctx* ctx, const AmmGeom& g, float* d_cent)
     rc = hip_check(ctx, hipGetLastError(), "ccs_prep_mfma_kernel launch");
     if (rc || !ccs_has_bf16(g)) return rc;
     float* bf = d_cent + ccs_bf16_offset(g);
-    hipLaunchKernelGGL(ccs_prep_bf16_kernel, dim3(g.CB_pad / 2), dim3(64), 0, ctx->stream, d_cent,
-                       reinterpret_cast<uint4*>(bf), bf + (size_t)(g.CB_pad / 2) * 3 * 64 * 4, g.CB, g.C);
+    uint4* aux_b = reinterpret_cast<uint4*>(bf);
+    float* cn16 = bf + (size_t)(g.CB_pad / 2) * ccs_bf16_nm(g.v) * 64 * 4;
+    const dim3 pg(g.CB_pad / 2), pb(64);
+    switch (g.v) {
+        case 2: hipLaunchKernelGGL(ccs_prep_bf16_kernel<2>, pg, pb, 0, ctx->stream, d_cent, aux_b, cn16, g.CB, g.C); break;
+        case 4: hipLaunchKernelGGL(ccs_prep_bf16_kernel<4>, pg, pb, 0, ctx->stream, d_cent, aux_b, cn16, g.CB, g.C); break;
+        default: hipLaunchKernelGGL(ccs_prep_bf16_kernel<8>, pg, pb, 0, ctx->stream, d_cent, aux_b, cn16, g.CB, g.C); break;
+    }
     return hip_check(ctx, hipGetLastError(), "ccs_prep_bf16_kernel launch");
 }
 
