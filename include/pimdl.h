@@ -222,6 +222,12 @@ PIMDL_API int pimdl_amm_get_geometry(const pimdl_amm* amm, pimdl_amm_geometry* g
  * (b) a ds_read_b128 loop that keeps every CU's LDS busy.  Either pointer may be NULL. */
 PIMDL_API int pimdl_diag_bandwidth(pimdl_ctx* ctx, uint64_t bytes, float* copy_gbps,
                                    float* lds_gbps);
+/* Checks on this device what the bf16-split closest-centroid search takes for granted about the
+ * matrix core: runs `trials` (1..4096) chains of three v_mfma_f32_32x32x16_bf16 on random operands of
+ * mixed magnitude and reports the largest |result - exact sum| in units of 2^-24 * sum|terms|.  The
+ * search kernel's margin allows 51 of these units (sub_vec_len 4); index_calculation itself
+ * (src/host/index_calc_host.cpp:8-53) has no counterpart of this: it is a property of this port. */
+PIMDL_API int pimdl_diag_mfma_error(pimdl_ctx* ctx, uint32_t trials, float* max_err_u);
 
 #ifdef __cplusplus
 }

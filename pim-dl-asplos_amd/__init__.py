@@ -28,7 +28,8 @@ EXPORTS = ["pimdl_init", "pimdl_destroy", "pimdl_last_error", "pimdl_set_stream"
            "pimdl_amm_create", "pimdl_amm_create_tuned", "pimdl_amm_destroy", "pimdl_amm_run", "pimdl_amm_run_debug",
            "pimdl_amm_profile", "pimdl_index_calculation", "pimdl_amm_index_calculation", "pimdl_lut_gather",
            "pimdl_amm_run_tiled", "pimdl_lut_gather_tiled", "pimdl_lutgen",
-           "pimdl_layer_norm", "pimdl_get_device_info", "pimdl_amm_get_geometry", "pimdl_diag_bandwidth"]
+           "pimdl_layer_norm", "pimdl_get_device_info", "pimdl_amm_get_geometry", "pimdl_diag_bandwidth",
+           "pimdl_diag_mfma_error"]
 
 
 class PimdlError(RuntimeError):
@@ -125,6 +126,7 @@ def lib():
     L.pimdl_get_device_info.argtypes = [vp, ctypes.POINTER(DeviceInfo)]
     L.pimdl_amm_get_geometry.argtypes = [vp, ctypes.POINTER(AmmGeometry)]
     L.pimdl_diag_bandwidth.argtypes = [vp, u64, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float)]
+    L.pimdl_diag_mfma_error.argtypes = [vp, ctypes.c_uint32, ctypes.POINTER(ctypes.c_float)]
     for name in EXPORTS:
         if name != "pimdl_last_error":
             getattr(L, name).restype = ctypes.c_int
@@ -182,6 +184,12 @@ class Context:
         self._check(lib().pimdl_diag_bandwidth(self._h, nbytes, ctypes.byref(c) if copy else None,
                                                ctypes.byref(l) if lds else None))
         return c.value, l.value
+
+    def diag_mfma_error(self, trials=256):
+        """Largest error of a chain of three bf16 MFMAs against the exact sum, in units of 2^-24 * sum|terms|."""
+        e = ctypes.c_float(0)
+        self._check(lib().pimdl_diag_mfma_error(self._h, trials, ctypes.byref(e)))
+        return e.value
 
     def index_calculation(self, x, centroids, n_stile=0, cb_mtile=0):
         """Context-level closest-centroid search: centroids are passed (and uploaded) per call."""

@@ -37,6 +37,11 @@
 // v for the FMAs whose partial sums stay below 2(XX+CN)).  Sum: (5v+5)u(XX+CN); the kernel uses
 // three times that.  Packing the id into the low IDX_BITS bits moves a value by less than
 // 2^IDX_BITS ulp, i.e. 2^(IDX_BITS-22) |value|, charged against the second-smallest value.
+#include <math.h>
+#include <string.h>
+
+#include <vector>
+
 #include "pimdl_internal.h"
 
 #include <stdlib.h>
@@ -1191,6 +1196,104 @@ int launch_ccs_bits(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d
 }
 
 }  // namespace
+
+// Measures what the bf16-split search assumes about the matrix core: a chain of three
+// v_mfma_f32_32x32x16_bf16 (48 products + the initial accumulator) against the exact sum, over random
+// operands whose pieces differ in magnitude like xh/xm/xl do.  Reports max |D - exact| / (u * sum|terms|).
+// The search kernel's bound allows 2.02 (12 v + NM) u per partial sum, i.e. 51 in this unit for v = 4.
+namespace {
+__global__ void mfma_error_kernel(const uint4* __restrict__ a, const uint4* __restrict__ b, const float* __restrict__ c,
+                                  float* __restrict__ d, int chain)
+{
+    const int l = threadIdx.x;
+    a += (size_t)blockIdx.x * chain * 64;
+    b += (size_t)blockIdx.x * chain * 64;
+    c += (size_t)blockIdx.x * 1024;
+    d += (size_t)blockIdx.x * 1024;
+    floatx16 acc;
+    for (int r = 0; r < 16; ++r) acc[r] = c[(8 * (r / 4) + 4 * (l / 32) + r % 4) * 32 + (l % 32)];
+    for (int m = 0; m < chain; ++m)
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[m * 64 + l]),
+                                                      __builtin_bit_cast(bf16x8, b[m * 64 + l]), acc, 0, 0, 0);
+    for (int r = 0; r < 16; ++r) d[(8 * (r / 4) + 4 * (l / 32) + r % 4) * 32 + (l % 32)] = acc[r];
+}
+}  // namespace
+
+int launch_diag_mfma_error(Ctx* ctx, uint32_t trials, float* max_err_u)
+{
+    constexpr int CHAIN = 3;
+    if (trials == 0 || trials > 4096) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_diag_mfma_error: trials must be in 1..4096");
+    std::vector<uint16_t> A((size_t)trials * CHAIN * 32 * 16), B((size_t)trials * CHAIN * 16 * 32);
+    std::vector<float> C((size_t)trials * 1024), D((size_t)trials * 1024);
+    uint64_t st = 0x9E3779B97F4A7C15ull;
+    auto next = [&]() {  // splitmix64
+        uint64_t z = (st += 0x9E3779B97F4A7C15ull);
+        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+        z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+        return z ^ (z >> 31);
+    };
+    auto unif = [&]() { return (float)((double)(next() >> 11) / 9007199254740992.0 * 2.0 - 1.0); };
+    auto to_bf16 = [](float f) { uint32_t u; memcpy(&u, &f, 4); return (uint16_t)(u >> 16); };
+    auto from_bf16 = [](uint16_t h) { uint32_t u = (uint32_t)h << 16; float f; memcpy(&f, &u, 4); return f; };
+    for (uint32_t t = 0; t < trials; ++t) {
+        const float small = ldexpf(1.0f, (int)(t % 5) * 6 - 24);
+        for (size_t i = 0; i < (size_t)CHAIN * 512; ++i) {
+            A[(size_t)t * CHAIN * 512 + i] = to_bf16(3.0f * unif() * ((next() & 1) ? 1.0f : small));
+            B[(size_t)t * CHAIN * 512 + i] = to_bf16(3.0f * unif() * ((next() & 3) ? 1.0f : small));
+        }
+        for (size_t i = 0; i < 1024; ++i) C[(size_t)t * 1024 + i] = 8.0f * unif();
+    }
+    std::vector<uint4> ha((size_t)trials * CHAIN * 64), hb((size_t)trials * CHAIN * 64);
+    for (uint32_t t = 0; t < trials; ++t)
+        for (int m = 0; m < CHAIN; ++m)
+            for (int l = 0; l < 64; ++l) {
+                uint16_t pa[8], pb[8];
+                for (int e = 0; e < 8; ++e) {
+                    const int kk = 8 * (l / 32) + e;
+                    pa[e] = A[((size_t)(t * CHAIN + m) * 32 + l % 32) * 16 + kk];
+                    pb[e] = B[((size_t)(t * CHAIN + m) * 16 + kk) * 32 + l % 32];
+                }
+                memcpy(&ha[(size_t)(t * CHAIN + m) * 64 + l], pa, 16);
+                memcpy(&hb[(size_t)(t * CHAIN + m) * 64 + l], pb, 16);
+            }
+    uint4 *da = nullptr, *db = nullptr;
+    float *dc = nullptr, *dd = nullptr;
+    int rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&da), ha.size() * 16), "hipMalloc(diag)");
+    if (!rc) rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&db), hb.size() * 16), "hipMalloc(diag)");
+    if (!rc) rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&dc), C.size() * 4), "hipMalloc(diag)");
+    if (!rc) rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&dd), D.size() * 4), "hipMalloc(diag)");
+    if (!rc) rc = hip_check(ctx, hipMemcpy(da, ha.data(), ha.size() * 16, hipMemcpyHostToDevice), "H2D diag");
+    if (!rc) rc = hip_check(ctx, hipMemcpy(db, hb.data(), hb.size() * 16, hipMemcpyHostToDevice), "H2D diag");
+    if (!rc) rc = hip_check(ctx, hipMemcpy(dc, C.data(), C.size() * 4, hipMemcpyHostToDevice), "H2D diag");
+    if (!rc) {
+        hipLaunchKernelGGL(mfma_error_kernel, dim3(trials), dim3(64), 0, ctx->stream, da, db, dc, dd, CHAIN);
+        rc = hip_check(ctx, hipGetLastError(), "mfma_error_kernel launch");
+    }
+    if (!rc) rc = hip_check(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+    if (!rc) rc = hip_check(ctx, hipMemcpy(D.data(), dd, D.size() * 4, hipMemcpyDeviceToHost), "D2H diag");
+    (void)hipFree(da);
+    (void)hipFree(db);
+    (void)hipFree(dc);
+    (void)hipFree(dd);
+    if (rc) return rc;
+    double worst = 0.0;
+    for (uint32_t t = 0; t < trials; ++t)
+        for (int i = 0; i < 32; ++i)
+            for (int j = 0; j < 32; ++j) {
+                double ex = C[(size_t)t * 1024 + i * 32 + j], sabs = fabs(ex);
+                for (int m = 0; m < CHAIN; ++m)
+                    for (int kk = 0; kk < 16; ++kk) {
+                        const double p = (double)from_bf16(A[((size_t)(t * CHAIN + m) * 32 + i) * 16 + kk]) *
+                                         (double)from_bf16(B[((size_t)(t * CHAIN + m) * 16 + kk) * 32 + j]);
+                        ex += p;
+                        sabs += fabs(p);
+                    }
+                const double e = fabs((double)D[(size_t)t * 1024 + i * 32 + j] - ex) / (5.9604644775390625e-8 * sabs);
+                if (e > worst) worst = e;
+            }
+    *max_err_u = (float)worst;
+    return PIMDL_OK;
+}
 
 // PIMDL_CCS_EXACT=1 in the environment switches the two-speed search off (every pair takes the
 // reference's scan); the results are the same by construction, so this is a debugging aid only.

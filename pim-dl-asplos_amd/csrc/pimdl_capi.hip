@@ -659,4 +659,13 @@ int pimdl_diag_bandwidth(pimdl_ctx* ctx, uint64_t bytes, float* copy_gbps, float
     return launch_diag(ctx, bytes, copy_gbps, lds_gbps);
 }
 
+int pimdl_diag_mfma_error(pimdl_ctx* ctx, uint32_t trials, float* max_err_u)
+{
+    if (!ctx) return PIMDL_ERR_INVALID;
+    if (!max_err_u) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_diag_mfma_error: null result pointer");
+    int rc = activate(ctx);
+    if (rc) return rc;
+    return launch_diag_mfma_error(ctx, trials, max_err_u);
+}
+
 }  // extern "C"

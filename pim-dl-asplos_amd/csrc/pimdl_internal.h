@@ -122,6 +122,7 @@ int launch_lut_quant(Ctx* ctx, const float* d_lut, int8_t* d_q, float* d_scales,
 int launch_layer_norm(Ctx* ctx, const float* d_x, const float* d_w, const float* d_b, const float* d_residual,
                       float* d_out, uint32_t n, uint32_t d, float eps);
 int launch_diag(Ctx* ctx, uint64_t bytes, float* copy_gbps, float* lds_gbps);
+int launch_diag_mfma_error(Ctx* ctx, uint32_t trials, float* max_err_u);
 
 uint32_t ccs_cb_per_wg(uint32_t v);  // codebooks one ccs workgroup covers (0: generic kernel)
 bool gather_rows_only();

@@ -311,6 +311,15 @@ def test_search_with_non_finite_values(ctx, v, C):
     amm.close()
 
 
+def test_matrix_core_rounding_stays_inside_the_search_margin(ctx):
+    """The bf16-split search accepts a winner only outside an error margin that assumes every addition of
+    the matrix core's chain (48 products + the initial accumulator) is within 2^-24 of the partial sum:
+    51 units of 2^-24 * sum|terms| for v = 4.  Measured on this device over 10^6 outputs with operand pieces
+    of mixed magnitude, the chain stays an order of magnitude inside that."""
+    worst = ctx.diag_mfma_error(1024)
+    assert 0.0 < worst < 12.0, worst
+
+
 def test_search_at_full_ffn2_shape(ctx):
     """N=8192, K=3072, v=4, 16 centroids: every index of the headline shape against the oracle,
     once with N(0,1) data and once with the reference driver's ranges."""
