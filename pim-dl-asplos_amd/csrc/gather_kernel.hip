@@ -54,6 +54,48 @@ struct Epilogue {
     const float* bias;    // [M] or nullptr
 };
 
+// How the items (column tile x token tile) of a gather are dealt to the 8 XCDs.  Workgroup b takes
+// positions b, b + grid, ... of the item sequence and the hardware places workgroups on the XCDs
+// round-robin, so (for a grid that is a multiple of 8) positions congruent mod 8 run on one XCD, each
+// with an L2 of its own.  XCD x = cx + col_split * tx then owns the column tiles congruent to cx mod
+// col_split and the token tiles congruent to tx mod tok_split (col_split * tok_split = 8), and its L2
+// fetches only that share of the LUT and of the index buffer instead of all of both.
+// col_split = 0: plain order, position p = column tile p / n_token_tiles, token tile p % n_token_tiles.
+struct XcdMap {
+    uint32_t col_split, tok_split, tok_per_xcd;  // tok_per_xcd = n_token_tiles / tok_split
+    __device__ __forceinline__ void decode(uint32_t p, uint32_t n_token_tiles, uint32_t& col, uint32_t& tok) const
+    {
+        if (col_split == 0) {
+            col = p / n_token_tiles;
+            tok = p % n_token_tiles;
+        } else {
+            const uint32_t x = p % 8, q = p / 8;
+            col = x % col_split + col_split * (q / tok_per_xcd);
+            tok = x / col_split + tok_split * (q % tok_per_xcd);
+        }
+    }
+};
+
+// Picks the split with the least L2 fill traffic: 8 * (lut_bytes / col_split + idx_bytes / tok_split).
+inline XcdMap choose_xcd_map(uint32_t n_col_tiles, uint32_t n_token_tiles, uint32_t grid, uint64_t lut_bytes,
+                             uint64_t idx_bytes)
+{
+    XcdMap best{0, 0, 0};
+    if (grid % 8 != 0) return best;
+    uint64_t best_cost = lut_bytes + idx_bytes / 8 + 1;  // plain order: every XCD reads the whole LUT
+    best_cost *= 8;
+    for (uint32_t cs = 8; cs >= 1; cs /= 2) {
+        const uint32_t ts = 8 / cs;
+        if (n_col_tiles % cs != 0 || n_token_tiles % ts != 0) continue;
+        const uint64_t cost = 8 * (lut_bytes / cs + idx_bytes / ts);
+        if (cost < best_cost) {
+            best_cost = cost;
+            best = XcdMap{cs, ts, n_token_tiles / ts};
+        }
+    }
+    return best;
+}
+
 constexpr int GATHER_WAVES = 8;
 constexpr int GATHER_THREADS = GATHER_WAVES * 64;
 
@@ -483,7 +525,7 @@ template <int TN, int TM>
 __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
     const uint8_t* __restrict__ idx, const int8_t* __restrict__ lut, float* __restrict__ out,
     int32_t* __restrict__ acc_out, uint32_t N, uint32_t M, uint32_t CB_pad, uint32_t idx_row_bytes,
-    uint32_t n_token_tiles, uint32_t n_items, Epilogue ep)
+    uint32_t n_token_tiles, uint32_t n_items, Epilogue ep, XcdMap xmap)
 {
     constexpr int OH_TOK_ITEM = oh_tok_item(TM);
     static_assert(TM == 4 || TM == 2, "a wave owns a whole or half a 64-token index block");
@@ -532,20 +574,22 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
     //          into [wave][word][64 tokens]; only the wave itself reads them back.
     // Addresses are kept as a wave-uniform 64-bit base (scalar registers) plus a 32-bit per-lane
     // offset, the form the copy instructions take directly.
+    auto col_of = [&](uint32_t p) { uint32_t c, t; xmap.decode(p, n_token_tiles, c, t); return c; };
+    auto tok_tile_of = [&](uint32_t p) { uint32_t c, t; xmap.decode(p, n_token_tiles, c, t); return t; };
     uint32_t lut_item = blockIdx.x, lut_s = 0, ix_item = blockIdx.x, ix_s = 0;
     const int8_t* dma_base;   // uniform: start of the slice at the LUT stream position
     const uint32_t dma_lane = wave * 1024 + lane * 16;
     const uint8_t* ix_base;   // uniform: the 256-byte block of index words at the index stream position
     uint32_t ix_lane_off;     // per lane: its token's word inside a block
     auto locate_lut = [&]() {
-        dma_base = lut + (size_t)(lut_item / n_token_tiles) * CB_pad * (WN * 16);
+        dma_base = lut + (size_t)col_of(lut_item) * CB_pad * (WN * 16);
     };
     // Index words live as [N/64][row words][64 tokens]: the word of a slice for this wave's 64 tokens
     // is one contiguous 256-byte block (see idx_offset).
     const uint32_t last_block = (N - 1) / 64;
     auto locate_ix = [&]() {
         // TM = 4: wave w owns block w of the tile; TM = 2: waves 2p and 2p+1 each copy block p and own half of it
-        uint32_t blk = ((ix_item % n_token_tiles) * OH_TOK_ITEM + wave * (TM * 16)) / 64;
+        uint32_t blk = (tok_tile_of(ix_item) * OH_TOK_ITEM + wave * (TM * 16)) / 64;
         if (blk > last_block) blk = last_block;  // clamp: results of such tokens are never stored
         ix_base = idx + (size_t)blk * idx_row_bytes * 64;
         ix_lane_off = lane * 4;
@@ -637,8 +681,8 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
         // registers for the whole kernel
         uint32_t je = j, ge = g;
         asm volatile("" : "+v"(je), "+v"(ge));
-        const uint32_t colblk = item / n_token_tiles;
-        const uint32_t tile_tok0 = (item % n_token_tiles) * OH_TOK_ITEM;
+        const uint32_t colblk = col_of(item);
+        const uint32_t tile_tok0 = tok_tile_of(item) * OH_TOK_ITEM;
         const uint32_t tok0 = tile_tok0 + wave * (TM * 16);
         const bool vec_store = (M % 4 == 0);
         const bool full = vec_store && !acc_out && tile_tok0 + OH_TOK_ITEM <= N && (colblk + 1) * WN <= M;
@@ -812,9 +856,11 @@ int launch_onehot_tm(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out,
     const uint32_t n_items = n_token_tiles * (a.g.M_pad / (16 * TN));
     uint32_t grid = ctx->prop.multiProcessorCount * 2;  // two workgroups per CU, see plan_geometry
     if (grid > n_items) grid = n_items;
+    const XcdMap xmap = choose_xcd_map(a.g.M_pad / (16 * TN), n_token_tiles, grid,
+                                       (uint64_t)a.g.CB_pad * 16 * a.g.M_pad, (uint64_t)n * a.g.idx_row_bytes);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(OH_THREADS), LDS, ctx->stream, d_idx,
                        reinterpret_cast<const int8_t*>(a.d_lut), d_out, d_acc, n, a.g.M, a.g.CB_pad,
-                       a.g.idx_row_bytes, n_token_tiles, n_items, ep);
+                       a.g.idx_row_bytes, n_token_tiles, n_items, ep, xmap);
     return hip_check(ctx, hipGetLastError(), "gather_onehot_kernel launch");
 }
 

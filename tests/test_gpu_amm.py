@@ -93,6 +93,28 @@ def test_ragged_shapes(ctx, N, K, v, C, M):
     check_i8(ctx, N + K + M, N, K, v, C, M)
 
 
+@pytest.mark.parametrize("N,M", [
+    (512, 768),     # 8 column tiles x 4 token tiles: one column tile per XCD
+    (1000, 380),    # 4 column tiles x 8 token tiles (last one ragged): columns over 4, tokens over 2
+    (2048, 192),    # 2 column tiles x 16 token tiles: columns over 2, tokens over 4
+    (4096, 96),     # 1 column tile x 32 token tiles: tokens over 8
+    (768, 768),     # 6 token tiles: no split divides, plain order
+])
+def test_every_item_is_computed_once_however_items_are_dealt_to_the_xcds(ctx, N, M):
+    """The one-hot gather deals (column tile, token tile) items to the 8 XCDs by a split chosen per shape;
+    a dropped or doubled item shows as wrong accumulators."""
+    x, cent, lut, bias = make_case(N + M, N, 128, 4, 16, M)
+    amm = ctx.amm(cent, lut, np.float32(0.01), bias, max_n=N, col_block=96)
+    out, idx, acc = amm.run_debug(x)
+    want_idx = oracle.index_calculation(x, cent, 4, threads=THREADS)
+    want_acc = oracle.gather_i8(want_idx, lut, threads=THREADS)
+    assert np.array_equal(idx, want_idx)
+    assert np.array_equal(acc, want_acc)
+    assert np.array_equal(out.view(np.uint32),
+                          oracle.dequant(want_acc, bias, 32, 0.01, 0.0, 0, threads=THREADS).view(np.uint32))
+    amm.close()
+
+
 def test_reference_driver_value_ranges_and_bias_modes(ctx):
     # uniform(-5,5) activations, uniform(-10,10) centroids, scale 0.1, bias 0.2 as in the shipped YAML
     check_i8(ctx, 7, 256, 128, 4, 16, 96, scale=0.1, lut_bias=0.2, bias_mode=0, dist="uniform")
