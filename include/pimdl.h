@@ -53,6 +53,15 @@ typedef enum pimdl_lut_dtype { PIMDL_LUT_I8 = 0, PIMDL_LUT_F32 = 1 } pimdl_lut_d
  *   PIMDL_BIAS_TIMES_CB   out = acc*scale + lut_bias*CB   + bias[f]   src/host/pim_lut_host.cpp:201 */
 typedef enum pimdl_bias_mode { PIMDL_BIAS_ONCE = 0, PIMDL_BIAS_TIMES_CB = 1 } pimdl_bias_mode;
 
+/* Function applied to every output element by the gather kernel's epilogue, after the bias.
+ *   PIMDL_ACT_NONE        out = y                                   amm_host as in the reference
+ *   PIMDL_ACT_GELU_TANH   out = 0.5 y (1 + tanh(sqrt(2/pi) (y + 0.044715 y^3)))
+ * The reference's layer applies GELU to the first feed-forward AMM's output in a pass of its own
+ * (ggml_gelu_inplace, src/host/transformer_layer.cpp:499-556); folding it into the epilogue saves
+ * one read and one write of the [N][ffn_hidden_dim] tensor.  fp32, within 1e-6 relative of the
+ * formula (evaluated as y / (1 + exp(-2u)), which does not cancel for negative y). */
+typedef enum pimdl_activation { PIMDL_ACT_NONE = 0, PIMDL_ACT_GELU_TANH = 1 } pimdl_activation;
+
 typedef struct pimdl_ctx pimdl_ctx; /* one device + one stream + scratch */
 typedef struct pimdl_amm pimdl_amm; /* one linear layer's centroids + LUT + bias, resident in HBM */
 
@@ -74,6 +83,7 @@ typedef struct pimdl_amm_desc {
                                    (the table is resident as fp32 integers, 4 bytes/entry). */
     uint32_t bias_mode;         /* pimdl_bias_mode */
     float lut_bias;             /* LUTParams.bias */
+    uint32_t activation;        /* pimdl_activation */
 } pimdl_amm_desc;
 
 /* Timing of the last profiled run, milliseconds on the device (HIP events on the context's

@@ -18,6 +18,7 @@ CSRC = os.path.join(_HERE, "csrc")
 
 LUT_I8, LUT_F32 = 0, 1
 BIAS_ONCE, BIAS_TIMES_CB = 0, 1
+ACT_NONE, ACT_GELU_TANH = 0, 1
 
 ERR_INVALID, ERR_UNSUPPORTED, ERR_HIP = -1, -2, -3
 STATUS = {0: "PIMDL_OK", -1: "PIMDL_ERR_INVALID", -2: "PIMDL_ERR_UNSUPPORTED", -3: "PIMDL_ERR_HIP",
@@ -43,7 +44,7 @@ class AmmDesc(ctypes.Structure):
                 ("sub_vec_len", ctypes.c_uint32), ("num_centroid", ctypes.c_uint32),
                 ("output_feature_len", ctypes.c_uint32), ("lut_dtype", ctypes.c_uint32),
                 ("scale_group", ctypes.c_uint32), ("bias_mode", ctypes.c_uint32),
-                ("lut_bias", ctypes.c_float)]
+                ("lut_bias", ctypes.c_float), ("activation", ctypes.c_uint32)]
 
 
 class AmmTiming(ctypes.Structure):
@@ -240,15 +241,17 @@ class Context:
         return y
 
     def amm(self, centroids, lut, scales=None, bias=None, max_n=8192, lut_bias=0.0, bias_mode=BIAS_ONCE,
-            scale_group=0, col_block=0):
-        """col_block: width of the gather kernel's column tile (0 = chosen by the library)."""
-        return Amm(self, centroids, lut, scales, bias, max_n, lut_bias, bias_mode, scale_group, col_block)
+            scale_group=0, col_block=0, activation=ACT_NONE):
+        """col_block: width of the gather kernel's column tile (0 = chosen by the library).
+        activation: ACT_GELU_TANH applies the tanh form of GELU to the output inside the gather's epilogue."""
+        return Amm(self, centroids, lut, scales, bias, max_n, lut_bias, bias_mode, scale_group, col_block, activation)
 
 
 class Amm:
     """One LUT-AMM operator resident in HBM."""
 
-    def __init__(self, ctx, centroids, lut, scales, bias, max_n, lut_bias, bias_mode, scale_group, col_block=0):
+    def __init__(self, ctx, centroids, lut, scales, bias, max_n, lut_bias, bias_mode, scale_group, col_block=0,
+                 activation=0):
         centroids = np.ascontiguousarray(centroids, np.float32)
         CB, C, v = centroids.shape
         lut = np.ascontiguousarray(lut)
@@ -256,7 +259,7 @@ class Amm:
         M = lut.shape[2]
         self.ctx, self.CB, self.C, self.v, self.K, self.M = ctx, CB, C, v, CB * v, M
         self.lut_dtype = LUT_I8 if lut.dtype == np.int8 else LUT_F32
-        desc = AmmDesc(max_n, CB * v, v, C, M, self.lut_dtype, scale_group, bias_mode, lut_bias)
+        desc = AmmDesc(max_n, CB * v, v, C, M, self.lut_dtype, scale_group, bias_mode, lut_bias, activation)
         if scales is not None:
             scales = np.ascontiguousarray(np.atleast_1d(scales), np.float32)
             want = (CB + scale_group - 1) // scale_group if (scale_group and self.lut_dtype == LUT_I8) else 1

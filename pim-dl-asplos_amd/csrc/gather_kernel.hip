@@ -52,6 +52,7 @@ struct Epilogue {
     float scale;
     float lut_bias_term;  // lut_bias or lut_bias*CB, already rounded to fp32 like the reference does
     const float* bias;    // [M] or nullptr
+    uint32_t act;         // pimdl_activation
 };
 
 // How the items (column tile x token tile) of a gather are dealt to the 8 XCDs.  Workgroup b takes
@@ -99,10 +100,26 @@ inline XcdMap choose_xcd_map(uint32_t n_col_tiles, uint32_t n_token_tiles, uint3
 constexpr int GATHER_WAVES = 8;
 constexpr int GATHER_THREADS = GATHER_WAVES * 64;
 
-__device__ __forceinline__ float dequant(int32_t acc, float scale, float lut_bias_term, float b)
+// The tanh form of GELU, 0.5 y (1 + tanh u) with u = sqrt(2/pi) (y + 0.044715 y^3), evaluated as
+// y * sigmoid(2u) = y / (1 + exp(-2u)): no cancellation of 1 + tanh u for negative y, exp overflow gives
+// y / inf = -0, and one v_exp_f32 plus one v_rcp_f32 (1 ulp each) keep it within 1e-6 relative.
+__device__ __forceinline__ float gelu_tanh(float y)
+{
+    constexpr float k0 = -2.0f * 0.7978845608028654f * 1.4426950408889634f;  // -2 sqrt(2/pi) log2(e)
+    constexpr float k1 = k0 * 0.044715f;
+    const float w = y * __builtin_fmaf(y * y, k1, k0);  // -2u log2(e)
+    return y * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(w));
+}
+
+__device__ __forceinline__ float activate(float y, uint32_t act)  // act is uniform over the launch
+{
+    return act == PIMDL_ACT_GELU_TANH ? gelu_tanh(y) : y;
+}
+
+__device__ __forceinline__ float dequant(int32_t acc, const Epilogue& ep, float b)
 {
     // ((float)acc * scale + lut_bias_term) + bias[f]   -- three separately rounded fp32 operations
-    return __fadd_rn(__fadd_rn(__fmul_rn((float)acc, scale), lut_bias_term), b);
+    return activate(__fadd_rn(__fadd_rn(__fmul_rn((float)acc, ep.scale), ep.lut_bias_term), b), ep.act);
 }
 
 template <int I, int N, class F>
@@ -336,10 +353,10 @@ __global__ __launch_bounds__(GATHER_THREADS, 4) void gather_i8_kernel(
                 acc[t][c] = (v4i){0, 0, 0, 0};
                 if (tok >= N || f >= M) continue;
                 float4 o;
-                o.x = dequant(a[0], ep.scale, ep.lut_bias_term, bv[c].x);
-                o.y = dequant(a[1], ep.scale, ep.lut_bias_term, bv[c].y);
-                o.z = dequant(a[2], ep.scale, ep.lut_bias_term, bv[c].z);
-                o.w = dequant(a[3], ep.scale, ep.lut_bias_term, bv[c].w);
+                o.x = dequant(a[0], ep, bv[c].x);
+                o.y = dequant(a[1], ep, bv[c].y);
+                o.z = dequant(a[2], ep, bv[c].z);
+                o.w = dequant(a[3], ep, bv[c].w);
                 if (vec_store) {  // M % 4 == 0 and f % 4 == 0: the whole float4 is in range and aligned
                     *reinterpret_cast<float4*>(out + (size_t)tok * M + f) = o;
                     if (acc_out) *reinterpret_cast<v4i*>(acc_out + (size_t)tok * M + f) = a;
@@ -708,10 +725,10 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
                 const v4i a = acc[t][c];
                 acc[t][c] = (v4i){0, 0, 0, 0};
                 float4 o;
-                o.x = dequant(a[0], ep.scale, ep.lut_bias_term, bv.x);
-                o.y = dequant(a[1], ep.scale, ep.lut_bias_term, bv.y);
-                o.z = dequant(a[2], ep.scale, ep.lut_bias_term, bv.z);
-                o.w = dequant(a[3], ep.scale, ep.lut_bias_term, bv.w);
+                o.x = dequant(a[0], ep, bv.x);
+                o.y = dequant(a[1], ep, bv.y);
+                o.z = dequant(a[2], ep, bv.z);
+                o.w = dequant(a[3], ep, bv.w);
                 if (full) {  // workgroup-uniform: every token and column of the tile exists
                     // streaming store: the output is not read again by this kernel
                     typedef float v4f __attribute__((ext_vector_type(4)));
@@ -895,7 +912,7 @@ __global__ __launch_bounds__(GF_THREADS) void gather_f32_kernel(const uint8_t* _
                                                                uint32_t idx_row_bytes,
                                                                const float* __restrict__ bias,
                                                                const float* __restrict__ scales,
-                                                               uint32_t CB, uint32_t group)
+                                                               uint32_t CB, uint32_t group, uint32_t act)
 {
     constexpr int FB = 4 * Q;             // columns per row
     constexpr int PITCH = 16 * Q + 16;    // bytes
@@ -1004,7 +1021,7 @@ __global__ __launch_bounds__(GF_THREADS) void gather_f32_kernel(const uint8_t* _
 #pragma unroll
         for (int i = 0; i < FB; ++i) {
             const uint32_t f = colblk * FB + i;
-            if (f < M) out[(size_t)tok * M + f] = __fadd_rn(GROUPED ? tot[i] : acc[i], bias ? bias[f] : 0.0f);
+            if (f < M) out[(size_t)tok * M + f] = activate(__fadd_rn(GROUPED ? tot[i] : acc[i], bias ? bias[f] : 0.0f), act);
         }
     }
 }
@@ -1053,7 +1070,7 @@ int launch_f32_impl(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, 
     dim3 grid((n + GF_THREADS - 1) / GF_THREADS, a.g.M_pad / (4 * Q));
     hipLaunchKernelGGL(kern, grid, dim3(GF_THREADS), LDS, ctx->stream, d_idx,
                        reinterpret_cast<const float*>(a.d_lut), d_out, n, a.g.M, a.g.CB_pad, a.g.idx_row_bytes,
-                       a.d_bias, a.d_scales, a.g.CB, a.desc.scale_group);
+                       a.d_bias, a.d_scales, a.g.CB, a.desc.scale_group, a.desc.activation);
     return hip_check(ctx, hipGetLastError(), "gather_f32_kernel launch");
 }
 
@@ -1094,6 +1111,7 @@ bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::s
     if (C < 1 || C > 256) { *why = "num_centroid must be in 1..256"; return false; }
     if (d.lut_dtype != PIMDL_LUT_I8 && d.lut_dtype != PIMDL_LUT_F32) { *why = "unknown lut_dtype"; return false; }
     if (d.bias_mode != PIMDL_BIAS_ONCE && d.bias_mode != PIMDL_BIAS_TIMES_CB) { *why = "unknown bias_mode"; return false; }
+    if (d.activation != PIMDL_ACT_NONE && d.activation != PIMDL_ACT_GELU_TANH) { *why = "unknown activation"; return false; }
     g->K = K; g->v = v; g->CB = K / v; g->C = C; g->M = M;
     g->CB_pad = (g->CB + 31) / 32 * 32;
     uint32_t ct = 8;
@@ -1195,6 +1213,7 @@ int launch_gather(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, in
         ep.scale = a.h_scale0;
         ep.lut_bias_term = a.desc.bias_mode == PIMDL_BIAS_TIMES_CB ? a.desc.lut_bias * (float)g.CB : a.desc.lut_bias;
         ep.bias = a.d_bias;
+        ep.act = a.desc.activation;
         if (g.gather_kind == 1) {
             switch (g.q) {
                 case 3: return launch_onehot<3>(ctx, a, d_idx, d_out, d_acc, n, ep);

@@ -150,13 +150,16 @@ def load_npz(path, params):
 class TransformerLayer:
     """One encoder layer resident on the GPU: six LUT-AMM operators and two LayerNorms."""
 
-    def __init__(self, ctx, pimdl, weights, params, fused_qkv=False, side=None):
-        """side: optional ((context, torch stream), (context, torch stream)) for the K and V projections.
+    def __init__(self, ctx, pimdl, weights, params, fused_qkv=False, side=None, fused_gelu=True):
+        """fused_gelu: GELU is applied by the first feed-forward operator's own epilogue instead of a pass of
+        its own over the [n][ffn_hidden_dim] tensor.
+        side: optional ((context, torch stream), (context, torch stream)) for the K and V projections.
         The three projections read the same input and are independent; at small batches each of them
         fills only half of the GPU, so running them on three streams overlaps them."""
         import torch
         self.ctx, self.params, self.torch = ctx, params, torch
         self.fused_qkv = fused_qkv
+        self.fused_gelu = fused_gelu
         self.side = None if fused_qkv else side
         n = params.n
         self.amm = {}
@@ -177,7 +180,9 @@ class TransformerLayer:
             if self.side and name in ("k", "v"):
                 owner = self.side[0 if name == "k" else 1][0]
             self.amm[name] = owner.amm(w["centroids"], w["lut"], np.float32(w["scale"]), w["bias"], max_n=n,
-                                       lut_bias=float(w.get("lut_bias", 0.0)), bias_mode=pimdl.BIAS_TIMES_CB)
+                                       lut_bias=float(w.get("lut_bias", 0.0)), bias_mode=pimdl.BIAS_TIMES_CB,
+                                       activation=pimdl.ACT_GELU_TANH if (fused_gelu and name == "ffn1")
+                                       else pimdl.ACT_NONE)
         dev = torch.device("cuda", torch.cuda.current_device())
         self.norm = {name: (torch.from_numpy(np.ascontiguousarray(weights[name]["weight"], np.float32)).to(dev),
                             torch.from_numpy(np.ascontiguousarray(weights[name]["bias"], np.float32)).to(dev))
@@ -233,8 +238,11 @@ class TransformerLayer:
         a = attn.permute(0, 2, 1, 3).reshape(n, p.token_dim).contiguous()
         o = self._run("o", a, n)
         h = self._norm_residual("attention_norm", o, x)
-        f1 = self._run("ffn1", h, n)
-        g = torch.nn.functional.gelu(f1, approximate="tanh")
+        if self.fused_gelu:
+            f1, g = None, self._run("ffn1", h, n)  # the pre-activation values never reach memory
+        else:
+            f1 = self._run("ffn1", h, n)
+            g = torch.nn.functional.gelu(f1, approximate="tanh")
         f2 = self._run("ffn2", g, n)
         y = self._norm_residual("ffn_norm", f2, h)
         if keep is not None:
@@ -245,7 +253,7 @@ class TransformerLayer:
 class Transformer:
     """layer_num encoder layers (transformer_model.cpp:13-49: each layer's output is the next one's input)."""
 
-    def __init__(self, ctx, pimdl, layers, params, fused_qkv=False, parallel_qkv=True):
+    def __init__(self, ctx, pimdl, layers, params, fused_qkv=False, parallel_qkv=True, fused_gelu=True):
         import torch
         self.side = None
         if parallel_qkv and not fused_qkv:
@@ -254,7 +262,7 @@ class Transformer:
                 c, st = pimdl.Context(torch.cuda.current_device()), torch.cuda.Stream()
                 c.set_stream(st.cuda_stream)
                 self.side.append((c, st))
-        self.layers = [TransformerLayer(ctx, pimdl, w, params, fused_qkv, self.side) for w in layers]
+        self.layers = [TransformerLayer(ctx, pimdl, w, params, fused_qkv, self.side, fused_gelu) for w in layers]
         self.params = params
 
     def close(self):

@@ -115,6 +115,38 @@ def test_every_item_is_computed_once_however_items_are_dealt_to_the_xcds(ctx, N,
     amm.close()
 
 
+@pytest.mark.parametrize("C,lut,group", [(16, "i8", 0), (32, "i8", 0), (16, "f32", 0), (16, "i8", 4)])
+def test_gelu_in_the_epilogue(ctx, C, lut, group):
+    """activation=ACT_GELU_TANH: same indices and accumulators, output = tanh-GELU of the plain output
+    (each of the gather kernels: matrix-core one-hot, byte adder, fp32 table, grouped scales)."""
+    N, K, v, M = 300, 128, 4, 200
+    x, cent, table, bias = make_case(C + group, N, K, v, C, M, lut)
+    CB = K // v
+    scales = None if lut == "f32" else (np.full((CB + group - 1) // group, 0.02, np.float32) if group else np.float32(0.02))
+    plain = ctx.amm(cent, table, scales, bias, max_n=N, scale_group=group)
+    fused = ctx.amm(cent, table, scales, bias, max_n=N, scale_group=group, activation=pimdl.ACT_GELU_TANH)
+    y = plain.run(x).astype(np.float64)
+    want = 0.5 * y * (1 + np.tanh(np.sqrt(2 / np.pi) * (y + 0.044715 * y ** 3)))
+    got = fused.run(x)
+    assert (np.abs(y) > 3).any() and (np.abs(y) < 0.1).any()  # both tails and the middle are exercised
+    np.testing.assert_allclose(got, want, rtol=2e-6, atol=1e-7)
+    if lut == "i8" and not group:
+        _, idx, acc = fused.run_debug(x)
+        _, idx0, acc0 = plain.run_debug(x)
+        assert np.array_equal(idx, idx0) and np.array_equal(acc, acc0)
+    # extreme inputs: -0 for very negative values (never NaN), identity for very positive ones
+    big = ctx.amm(cent, table, scales, np.where(np.arange(M) % 2 == 0, 1e6, -1e6).astype(np.float32), max_n=N,
+                  scale_group=group, activation=pimdl.ACT_GELU_TANH)
+    raw = ctx.amm(cent, table, scales, np.where(np.arange(M) % 2 == 0, 1e6, -1e6).astype(np.float32), max_n=N,
+                  scale_group=group)
+    yb, y0 = big.run(x), raw.run(x)
+    assert np.array_equal(yb[:, 0::2], y0[:, 0::2]) and not yb[:, 1::2].any() and not np.isnan(yb).any()
+    for a in (plain, fused, big, raw):
+        a.close()
+    with pytest.raises(pimdl.PimdlError):
+        ctx.amm(cent, table, scales, bias, max_n=N, scale_group=group, activation=7)
+
+
 def test_reference_driver_value_ranges_and_bias_modes(ctx):
     # uniform(-5,5) activations, uniform(-10,10) centroids, scale 0.1, bias 0.2 as in the shipped YAML
     check_i8(ctx, 7, 256, 128, 4, 16, 96, scale=0.1, lut_bias=0.2, bias_mode=0, dist="uniform")
