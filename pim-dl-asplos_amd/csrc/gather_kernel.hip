@@ -1087,8 +1087,8 @@ int launch_f32(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, uint3
 // the largest tables; two slices must fit the 160 KB LDS.  fp32: rows of 16 floats (Q=4).
 //   C_T   int8 (Q, GQ) -> slice bytes        fp32 (Q, GS) -> slice bytes
 //   8     (4, 8)  20 KB                      (4, 32) 20 KB
-//   16    (4, 8)  40 KB                      (4, 32) 40 KB
-//   32    (4, 4)  40 KB                      (4, 16) 40 KB
+//   16    (4, 8)  40 KB                      (4, 16) 20 KB
+//   32    (4, 4)  40 KB                      (4, 8)  20 KB
 //   64    (4, 2)  40 KB                      (4, 8)  40 KB
 //   128   (2, 2)  48 KB                      (2, 8)  48 KB
 //   256   (2, 1)  48 KB                      (2, 4)  48 KB
@@ -1190,7 +1190,7 @@ bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::s
         g->tokens_per_wg = GATHER_WAVES * 2 * 16;
     } else {
         g->gq = 0;
-        g->cb_per_slice = ct <= 16 ? 32 : ct == 32 ? 16 : ct <= 128 ? 8 : 4;
+        g->cb_per_slice = ct == 8 ? 32 : ct == 16 ? 16 : ct <= 128 ? 8 : 4;
         g->col_block = 4 * g->q;
         g->gather_threads = GF_THREADS;
         g->tokens_per_wg = GF_THREADS;
@@ -1239,8 +1239,8 @@ int launch_gather(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, in
     } else {
         switch (g.C_tile) {
             case 8: return launch_f32<8, 4, 32, 4>(ctx, a, d_idx, d_out, n);
-            case 16: return launch_f32<16, 4, 32, 4>(ctx, a, d_idx, d_out, n);
-            case 32: return launch_f32<32, 4, 16, 8>(ctx, a, d_idx, d_out, n);
+            case 16: return launch_f32<16, 4, 16, 4>(ctx, a, d_idx, d_out, n);
+            case 32: return launch_f32<32, 4, 8, 8>(ctx, a, d_idx, d_out, n);
             case 64: return launch_f32<64, 4, 8, 8>(ctx, a, d_idx, d_out, n);
             case 128: return launch_f32<128, 2, 8, 8>(ctx, a, d_idx, d_out, n);
             case 256: return launch_f32<256, 2, 4, 8>(ctx, a, d_idx, d_out, n);
