@@ -76,7 +76,11 @@ inline size_t ccs_aux_a_floats(const AmmGeom& g)
 
 // bf16-split search (v = 4, C <= 16): offset in floats of its operands behind everything else, and
 // their size.  The offset is rounded up to 16 bytes (uint4 operand images).
-inline bool ccs_has_bf16(const AmmGeom& g) { return (g.v == 2 || g.v == 4 || g.v == 8) && g.C <= 16; }
+inline bool ccs_has_bf16(const AmmGeom& g) { return (g.v == 2 || g.v == 4 || g.v == 8) && g.C <= 32; }
+// 17..32 centroids: a codebook fills all 32 rows of the matrix instruction by itself ("wide"); the operand
+// images are then per codebook instead of per pair of codebooks
+inline bool ccs_bf16_wide(const AmmGeom& g) { return g.C > 16; }
+inline size_t ccs_bf16_units(const AmmGeom& g) { return ccs_bf16_wide(g) ? g.CB_pad : g.CB_pad / 2; }
 // MFMAs (16 K-slots each) per codebook pair: 2 codebooks x v dims x 6 cross products
 constexpr uint32_t ccs_bf16_nm(uint32_t v) { return (12 * v + 15) / 16; }
 inline size_t ccs_bf16_offset(const AmmGeom& g)
@@ -86,7 +90,7 @@ inline size_t ccs_bf16_offset(const AmmGeom& g)
 }
 inline size_t ccs_bf16_floats(const AmmGeom& g)
 {
-    return ccs_has_bf16(g) ? (size_t)(g.CB_pad / 2) * ccs_bf16_nm(g.v) * 64 * 4 + (size_t)g.CB_pad * 16 : 0;
+    return ccs_has_bf16(g) ? ccs_bf16_units(g) * ccs_bf16_nm(g.v) * 64 * 4 + ccs_bf16_units(g) * 2 * 16 : 0;
 }
 
 template <int N, typename F>
@@ -348,11 +352,12 @@ __global__ __launch_bounds__(CCS_THREADS) void ccs_kernel(const float* __restric
 // each below 2(XX+CN): together with the reference chain's 2(v+2)u(XX+CN) that is below
 // (5v+8)u(XX+CN); the kernel uses twice that.
 // =============================================================================================
-template <int V>
+template <int V, bool WIDE = false>
 struct CcsMfmaShape {
     static constexpr int TILE_TOKENS = 128;
     static constexpr int CBW = 16;                         // codebooks per tile: 2 pairs per wave
-    static constexpr int TF = CBW * V;                     // floats per tile row
+    static constexpr int RCB = WIDE ? CBW / 2 : CBW;       // wide: a "pair" is the two 16-centroid halves of one codebook
+    static constexpr int TF = RCB * V;                     // floats per tile row
     static constexpr int PITCH = TF + 4;                   // +16 B: odd number of 16-byte units
     static constexpr int NQ = V + 1;                       // MFMAs (K = 2 each) per item
     static constexpr int TG = TILE_TOKENS / 32;            // 32-token groups
@@ -640,7 +645,9 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 //            {ch, cm, ch, cm, cl, ch} of -2c against the search kernel's {xh, xh, xm, xm, xh, xl};
 //   DL == 1: three registers for the one dim, (ch | cm), (ch | cm), (cl | ch) against (xh | xh), (xm | xm), (xh | xl).
 // Rows of the other codebook, and registers past 6*DL, hold zeros.
-template <uint32_t V>
+// WIDE (17..32 centroids): "pair" p is codebook p alone, its half h holds centroids 16h .. 16h+15, and both
+// halves meet the same sub-vector (the search kernel feeds the activations of codebook p to both).
+template <uint32_t V, bool WIDE>
 __global__ void ccs_prep_bf16_kernel(const float* __restrict__ cent, uint4* __restrict__ aux_b,
                                      float* __restrict__ cn16, uint32_t CB, uint32_t C)
 {
@@ -648,9 +655,10 @@ __global__ void ccs_prep_bf16_kernel(const float* __restrict__ cent, uint4* __re
     const uint32_t pair = blockIdx.x, lane = threadIdx.x;
     const uint32_t i = lane & 31, kh = lane >> 5;
     const uint32_t h = (i >> 2) & 1, r = (i & 3) + 4 * (i >> 3);
-    const uint32_t cb = 2 * pair + h;
-    const bool real = (cb < CB) && (r < C);
-    const float* cp = cent + ((size_t)cb * C + r) * V;
+    const uint32_t cb = WIDE ? pair : 2 * pair + h;
+    const uint32_t cid = WIDE ? 16 * h + r : r;  // centroid of row i
+    const bool real = (cb < CB) && (cid < C);
+    const float* cp = cent + ((size_t)cb * C + cid) * V;
     uint32_t pc[DL][3];  // bf16 pieces ch, cm, cl of -2c for the lane's dims
     for (uint32_t d = 0; d < DL; ++d) {
         const float a = real ? -2.0f * cp[DL * kh + d] : 0.0f;
@@ -682,7 +690,7 @@ __global__ void ccs_prep_bf16_kernel(const float* __restrict__ cent, uint4* __re
         aux_b[((size_t)pair * NM + m) * 64 + lane] = make_uint4(w[0], w[1], w[2], w[3]);
     }
     if (kh == 0) {
-        float cn = (float)r;  // a padded codebook scores r against centroid r: index 0 with a margin of 1
+        float cn = (float)cid;  // a padded codebook scores r against centroid r: index 0 with a margin of 1
         if (real) {
             cn = 0.0f;
             for (uint32_t t = 0; t < V; ++t) cn = fmaf(cp[t], cp[t], cn);
@@ -693,7 +701,7 @@ __global__ void ccs_prep_bf16_kernel(const float* __restrict__ cent, uint4* __re
     }
 }
 
-template <int V>
+template <int V, bool WIDE>
 __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* __restrict__ x,
                                                                  const float* __restrict__ cent,
                                                                  const uint4* __restrict__ aux_b,
@@ -704,8 +712,9 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
                                                                  uint32_t idx_row_bytes, int idx_tiled, int vec_ok,
                                                                  uint32_t tiles_cb, uint32_t total_tiles, uint32_t num_cus)
 {
-    using S = CcsMfmaShape<V>;
-    constexpr int TF = S::TF, PITCH = S::PITCH, TT = S::TILE_TOKENS, CBW = S::CBW, TG = S::TG;
+    using S = CcsMfmaShape<V, WIDE>;
+    constexpr int TF = S::TF, PITCH = S::PITCH, TT = S::TILE_TOKENS, CBW = S::CBW, TG = S::TG, RCB = S::RCB;
+    constexpr int XSTEP = WIDE ? V : 2 * V;  // activation floats per pair
     constexpr int NM = (int)ccs_bf16_nm(V);  // MFMAs per item: 2 codebooks x v dims x 6 cross products, 16 K-slots each
     constexpr int DL = V / 2;                // dims of each codebook this lane supplies
     constexpr int ITEMS = S::ITEMS;
@@ -741,7 +750,7 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
         }
     };
     // operands of this lane inside the tile: row of token (32 tg + j), columns of pair (2 wave + pl)
-    const float* brow0 = tile + j * PITCH + 2 * wave * 2 * V;
+    const float* brow0 = tile + j * PITCH + 2 * wave * XSTEP;
 
     float4 pf[PASSES];
     if (blockIdx.x < total_tiles) fetch(pf, blockIdx.x);
@@ -773,11 +782,11 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
         // loads complete in order, so a later load would have to wait for the prefetch from HBM
         float cmax[2];
 #pragma unroll
-        for (int pl = 0; pl < 2; ++pl) cmax[pl] = cnmax_pad[2 * (pair0 + pl) + h];
+        for (int pl = 0; pl < 2; ++pl) cmax[pl] = cnmax_pad[WIDE ? pair0 + pl : 2 * (pair0 + pl) + h];
         // raw centroids of the tile's codebooks, only read by exact replays
-        const uint32_t cb_here = (CB - tcb * CBW < (uint32_t)CBW) ? CB - tcb * CBW : (uint32_t)CBW;
+        const uint32_t cb_here = (CB - tcb * RCB < (uint32_t)RCB) ? CB - tcb * RCB : (uint32_t)RCB;
         const uint32_t cent_fl = cb_here * C * V;
-        const float* csrc = cent + (size_t)tcb * CBW * C * V;  // 16-byte aligned: CBW * V * 4 bytes per c
+        const float* csrc = cent + (size_t)tcb * RCB * C * V;  // 16-byte aligned: RCB * V * 4 bytes per c
 #pragma unroll
         for (int i = 0; i < PASSES; ++i)
             *reinterpret_cast<float4*>(&tile[(fr0 + i * ROWS_PER_PASS) * PITCH + 4 * fq]) = pf[i];
@@ -797,11 +806,11 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
         // accumulators start from |c|^2.  xx_out: |x|^2 over the lane's own codebook (for the bound).
         auto scores = [&](floatx16& acc, float& xx_out, int it) {
             const int pl = it / TG, tg = it % TG;
-            const float* brow = brow0 + tg * 32 * PITCH + pl * 2 * V;
+            const float* brow = brow0 + tg * 32 * PITCH + pl * XSTEP;
             float xs[2][DL];
 #pragma unroll
             for (int cbh = 0; cbh < 2; ++cbh) {
-                const float* src = brow + cbh * V + DL * h;
+                const float* src = brow + (WIDE ? 0 : cbh * V) + DL * h;
                 if constexpr (DL == 1) {
                     xs[cbh][0] = src[0];
                 } else if constexpr (DL == 2) {
@@ -905,9 +914,21 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
             }
             const float a1 = vmin3(lo[0], lo[1], lo[2]), a2 = __builtin_amdgcn_fmed3f(lo[0], lo[1], lo[2]);
             const float b1 = vmin3(lo[3], lo[4], key[15]), b2 = __builtin_amdgcn_fmed3f(lo[3], lo[4], key[15]);
-            const float m1 = vmin(a1, b1);
-            const float m2 = vmin3(vmin3(md[0], md[1], md[2]), vmin3(md[3], md[4], vmax(a1, b1)), vmin(a2, b2));
-            const uint32_t bi = __float_as_uint(m1) & 15u;
+            float m1 = vmin(a1, b1);
+            float m2 = vmin3(vmin3(md[0], md[1], md[2]), vmin3(md[3], md[4], vmax(a1, b1)), vmin(a2, b2));
+            uint32_t bi = __float_as_uint(m1) & 15u;
+            if constexpr (WIDE) {
+                // the other 16 centroids of the codebook were searched by lane l ^ 32: both lanes merge the
+                // two (smallest, second smallest) pairs and reach the same verdict.  Equal tagged minima
+                // give m2 == m1, which fails the margin test.
+                const auto s1 = __builtin_amdgcn_permlane32_swap(__float_as_uint(m1), __float_as_uint(m1), false, false);
+                const auto s2 = __builtin_amdgcn_permlane32_swap(__float_as_uint(m2), __float_as_uint(m2), false, false);
+                const float m1lo = __uint_as_float(s1[0]), m1hi = __uint_as_float(s1[1]);
+                const float m2lo = __uint_as_float(s2[0]), m2hi = __uint_as_float(s2[1]);
+                m1 = vmin(m1lo, m1hi);
+                m2 = vmin3(vmax(m1lo, m1hi), m2lo, m2hi);
+                bi = (__float_as_uint(m1) & 15u) | (m1hi < m1lo ? 16u : 0u);
+            }
             const float mag = xx + cmax[pl];
             // 2 * [ (v+1)u (|c|^2) + 16u (omitted products) + 2.02 (12v + NM) u (that many additions, each
             //       within u of a partial sum below 2.02 mag) + 2(v+2)u (the reference's own chain) ]
@@ -918,7 +939,10 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
             // NaN anywhere makes a compare false, which counts as "not safe"
             const bool safe = ((m2 - m1) > thr) && (mag < 1e36f);
             need |= (safe ? 0u : 1u) << it;
-            words[tg / 2] |= bi << (16 * (tg % 2) + 8 * pl + 4 * h);
+            if constexpr (WIDE)
+                words[tg / 2] |= (h == 0 ? bi : 0u) << (16 * (tg % 2) + 8 * pl);  // one byte per codebook
+            else
+                words[tg / 2] |= bi << (16 * (tg % 2) + 8 * pl + 4 * h);
             if constexpr (it + 1 < ITEMS) {
                 acc_cur = acc_nxt;
                 xx_cur = xx_nxt;
@@ -932,10 +956,10 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
             for (int it = 0; it < ITEMS; ++it) {
                 if (!((need >> it) & 1u)) continue;
                 const int pl = it / TG, tg = it % TG;
-                const uint32_t cbl = 2 * (2 * wave + pl) + h;
+                const uint32_t cbl = WIDE ? 2 * wave + pl : 2 * (2 * wave + pl) + h;  // codebook within the tile
                 uint32_t bi = 0;
-                if (tcb * CBW + cbl < CB) {
-                    const float* xo = brow0 + tg * 32 * PITCH + pl * 2 * V + V * h;
+                if (tcb * RCB + cbl < CB) {
+                    const float* xo = brow0 + tg * 32 * PITCH + pl * XSTEP + (WIDE ? 0 : V * h);
                     const float* cp = cst + cbl * C * V;
                     float best = 0.0f;
 #pragma nounroll
@@ -952,11 +976,14 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
                         bi = take ? c : bi;
                     }
                 }
-                const uint32_t sh = 16 * (tg % 2) + 8 * pl + 4 * h;
+                // wide: both lanes of the pair replay all of the codebook's centroids; lane h = 0 keeps the byte
+                const uint32_t sh = WIDE ? 16 * (tg % 2) + 8 * pl : 16 * (tg % 2) + 8 * pl + 4 * h;
+                const uint32_t keep_mask = WIDE ? 255u : 15u;
+                if (WIDE && h != 0) bi = 0;
                 uint32_t w = words[0];
 #pragma unroll
                 for (int i = 1; i < TG / 2; ++i) w = (tg / 2 == i) ? words[i] : w;
-                w = (w & ~(15u << sh)) | (bi << sh);
+                w = (w & ~(keep_mask << sh)) | (bi << sh);
 #pragma unroll
                 for (int i = 0; i < TG / 2; ++i) words[i] = (tg / 2 == i) ? w : words[i];
             }
@@ -1132,16 +1159,16 @@ static bool ccs_f32_only()
     return v;
 }
 
-template <int V>
+template <int V, bool WIDE>
 int launch_ccs_bf16(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_cent, uint8_t* d_idx, uint32_t n)
 {
-    using S = CcsMfmaShape<V>;
-    const uint32_t tiles_cb = g.CB_pad / S::CBW;  // CB_pad is a multiple of 32
+    using S = CcsMfmaShape<V, WIDE>;
+    const uint32_t tiles_cb = g.CB_pad / S::RCB;  // CB_pad is a multiple of 32
     const uint64_t total64 = (uint64_t)((n + S::TILE_TOKENS - 1) / S::TILE_TOKENS) * tiles_cb;
     if (total64 > 0xFFFFFFFFull) return set_error(ctx, PIMDL_ERR_INVALID, "ccs: too many tiles");
     const uint32_t total = (uint32_t)total64;
     int per_cu = 0;  // persistent grid: exactly the workgroups that are resident at once
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, ccs_bf16_kernel<V>, CCS_THREADS, 0) != hipSuccess || per_cu < 1) {
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, ccs_bf16_kernel<V, WIDE>, CCS_THREADS, 0) != hipSuccess || per_cu < 1) {
         (void)hipGetLastError();
         per_cu = 1;
     }
@@ -1153,8 +1180,8 @@ int launch_ccs_bf16(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d
     const float* cnmax_pad = cnmax + g.CB + (size_t)(g.CB_pad / 2) * (g.v + 1) * 64;
     const float* bf = d_cent + ccs_bf16_offset(g);
     const uint4* aux_b = reinterpret_cast<const uint4*>(bf);
-    const float* cn16 = bf + (size_t)(g.CB_pad / 2) * ccs_bf16_nm(V) * 64 * 4;
-    hipLaunchKernelGGL(ccs_bf16_kernel<V>, grid, dim3(CCS_THREADS), 0, ctx->stream, d_x, d_cent, aux_b, cn16, cnmax_pad,
+    const float* cn16 = bf + ccs_bf16_units(g) * ccs_bf16_nm(V) * 64 * 4;
+    hipLaunchKernelGGL((ccs_bf16_kernel<V, WIDE>), grid, dim3(CCS_THREADS), 0, ctx->stream, d_x, d_cent, aux_b, cn16, cnmax_pad,
                        d_idx, n, g.K, g.CB, g.C, g.idx_row_bytes, (int)g.idx_tiled, vec_ok, tiles_cb, total,
                        (uint32_t)ctx->prop.multiProcessorCount);
     return hip_check(ctx, hipGetLastError(), "ccs_bf16_kernel launch");
@@ -1163,12 +1190,20 @@ int launch_ccs_bf16(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d
 template <int IDX_BITS>
 int launch_ccs_bits(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_cent, uint8_t* d_idx, uint32_t n)
 {
+    if (IDX_BITS == 8 && g.C <= 32 && !ccs_exact_only() && !ccs_f32_only()) {
+        switch (g.v) {
+            case 2: return launch_ccs_bf16<2, true>(ctx, g, d_x, d_cent, d_idx, n);
+            case 4: return launch_ccs_bf16<4, true>(ctx, g, d_x, d_cent, d_idx, n);
+            case 8: return launch_ccs_bf16<8, true>(ctx, g, d_x, d_cent, d_idx, n);
+            default: break;
+        }
+    }
     if (IDX_BITS == 4 && !ccs_exact_only()) {
         if (!ccs_f32_only()) {
             switch (g.v) {
-                case 2: return launch_ccs_bf16<2>(ctx, g, d_x, d_cent, d_idx, n);
-                case 4: return launch_ccs_bf16<4>(ctx, g, d_x, d_cent, d_idx, n);
-                case 8: return launch_ccs_bf16<8>(ctx, g, d_x, d_cent, d_idx, n);
+                case 2: return launch_ccs_bf16<2, false>(ctx, g, d_x, d_cent, d_idx, n);
+                case 4: return launch_ccs_bf16<4, false>(ctx, g, d_x, d_cent, d_idx, n);
+                case 8: return launch_ccs_bf16<8, false>(ctx, g, d_x, d_cent, d_idx, n);
                 default: break;
             }
         }
@@ -1326,13 +1361,18 @@ int launch_ccs_prep(Ctx* ctx, const AmmGeom& g, float* d_cent)
     if (rc || !ccs_has_bf16(g)) return rc;
     float* bf = d_cent + ccs_bf16_offset(g);
     uint4* aux_b = reinterpret_cast<uint4*>(bf);
-    float* cn16 = bf + (size_t)(g.CB_pad / 2) * ccs_bf16_nm(g.v) * 64 * 4;
-    const dim3 pg(g.CB_pad / 2), pb(64);
+    float* cn16 = bf + ccs_bf16_units(g) * ccs_bf16_nm(g.v) * 64 * 4;
+    const dim3 pg((uint32_t)ccs_bf16_units(g)), pb(64);
+    const bool wide = ccs_bf16_wide(g);
+#define PIMDL_PREP_BF16(V_)                                                                                        \
+    if (wide) hipLaunchKernelGGL((ccs_prep_bf16_kernel<V_, true>), pg, pb, 0, ctx->stream, d_cent, aux_b, cn16, g.CB, g.C); \
+    else hipLaunchKernelGGL((ccs_prep_bf16_kernel<V_, false>), pg, pb, 0, ctx->stream, d_cent, aux_b, cn16, g.CB, g.C);
     switch (g.v) {
-        case 2: hipLaunchKernelGGL(ccs_prep_bf16_kernel<2>, pg, pb, 0, ctx->stream, d_cent, aux_b, cn16, g.CB, g.C); break;
-        case 4: hipLaunchKernelGGL(ccs_prep_bf16_kernel<4>, pg, pb, 0, ctx->stream, d_cent, aux_b, cn16, g.CB, g.C); break;
-        default: hipLaunchKernelGGL(ccs_prep_bf16_kernel<8>, pg, pb, 0, ctx->stream, d_cent, aux_b, cn16, g.CB, g.C); break;
+        case 2: PIMDL_PREP_BF16(2) break;
+        case 4: PIMDL_PREP_BF16(4) break;
+        default: PIMDL_PREP_BF16(8) break;
     }
+#undef PIMDL_PREP_BF16
     return hip_check(ctx, hipGetLastError(), "ccs_prep_bf16_kernel launch");
 }
 

@@ -88,6 +88,9 @@ def test_sweep_sub_vector_length_and_centroids(ctx, v, C):
     (513, 12, 3, 7, 33),     # sub_vec_len with no specialised kernel
     (64, 10, 5, 20, 18),     # generic v, 8-bit indices, K % 4 != 0
     (100, 6, 2, 16, 64),     # CB=3 (odd), K % 4 != 0: scalar activation loads
+    (300, 44, 4, 20, 40),    # 17..32 centroids on the matrix-core search: ids past C never win
+    (129, 18, 2, 17, 24),    # same, v=2, CB=9
+    (200, 72, 8, 31, 50),    # same, v=8
 ])
 def test_ragged_shapes(ctx, N, K, v, C, M):
     check_i8(ctx, N + K + M, N, K, v, C, M)
