@@ -904,7 +904,7 @@ int launch_onehot(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, in
 // ---------------------------------------------------------------------------------------------
 constexpr int GF_THREADS = 256;
 
-template <int C_T, int Q, int GS, int IDX_BITS, bool GROUPED>
+template <int C_T, int Q, int GS, int IDX_BITS, bool GROUPED, int TPL>
 __global__ __launch_bounds__(GF_THREADS) void gather_f32_kernel(const uint8_t* __restrict__ idx,
                                                                const float* __restrict__ lut,
                                                                float* __restrict__ out, uint32_t N,
@@ -925,23 +925,32 @@ __global__ __launch_bounds__(GF_THREADS) void gather_f32_kernel(const uint8_t* _
     static_assert(IDX_BYTES % 4 == 0, "index fetch is in dwords");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    const uint32_t tok = blockIdx.x * GF_THREADS + threadIdx.x;
-    const uint32_t tokc = tok < N ? tok : N - 1;
+    // TPL tokens per lane: the staged slice serves TPL * 256 tokens, so the table is streamed from L2
+    // 1/TPL as often
+    uint32_t tok[TPL];
+#pragma unroll
+    for (int t = 0; t < TPL; ++t) tok[t] = (blockIdx.x * TPL + t) * GF_THREADS + threadIdx.x;
     const uint32_t colblk = blockIdx.y;
     const uint32_t nslices = CB_pad / GS;
     const uint4* __restrict__ lut_blk = reinterpret_cast<const uint4*>(lut) + (size_t)colblk * CB_pad * C_T * Q;
-    const uint32_t* idx_row = reinterpret_cast<const uint32_t*>(idx + (size_t)tokc * idx_row_bytes);
+    const uint32_t* idx_row[TPL];
+#pragma unroll
+    for (int t = 0; t < TPL; ++t)
+        idx_row[t] = reinterpret_cast<const uint32_t*>(idx + (size_t)(tok[t] < N ? tok[t] : N - 1) * idx_row_bytes);
 
-    float acc[FB];
+    float acc[TPL][FB];
+    float tot[TPL][GROUPED ? FB : 1];
 #pragma unroll
-    for (int i = 0; i < FB; ++i) acc[i] = 0.0f;
-    float tot[GROUPED ? FB : 1];
+    for (int t = 0; t < TPL; ++t) {
 #pragma unroll
-    for (int i = 0; i < (GROUPED ? FB : 1); ++i) tot[i] = 0.0f;
+        for (int i = 0; i < FB; ++i) acc[t][i] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < (GROUPED ? FB : 1); ++i) tot[t][i] = 0.0f;
+    }
     uint32_t cb = 0, in_group = 0, gi = 0;  // workgroup-uniform position in the codebook sequence
 
     uint4 stage[UPT];
-    uint32_t idx_cur[IDX_WORDS], idx_nxt[IDX_WORDS];
+    uint32_t idx_cur[TPL][IDX_WORDS], idx_nxt[TPL][IDX_WORDS];
 #define PIMDL_FETCH_SLICE(S)                                                                        \
     {                                                                                               \
         const uint4* src_ = lut_blk + (size_t)(S) * SLICE_UNITS;                                    \
@@ -964,7 +973,9 @@ __global__ __launch_bounds__(GF_THREADS) void gather_f32_kernel(const uint8_t* _
     }
     PIMDL_FETCH_SLICE(0)
 #pragma unroll
-    for (int w = 0; w < IDX_WORDS; ++w) idx_cur[w] = idx_row[w];
+    for (int t = 0; t < TPL; ++t)
+#pragma unroll
+        for (int w = 0; w < IDX_WORDS; ++w) idx_cur[t][w] = idx_row[t][w];
     PIMDL_COMMIT_SLICE(0)
     __syncthreads();
 
@@ -973,35 +984,44 @@ __global__ __launch_bounds__(GF_THREADS) void gather_f32_kernel(const uint8_t* _
         const uint32_t sn = s + 1 < nslices ? s + 1 : s;
         PIMDL_FETCH_SLICE(sn)
 #pragma unroll
-        for (int w = 0; w < IDX_WORDS; ++w) idx_nxt[w] = idx_row[sn * IDX_WORDS + w];
+        for (int t = 0; t < TPL; ++t)
+#pragma unroll
+            for (int w = 0; w < IDX_WORDS; ++w) idx_nxt[t][w] = idx_row[t][sn * IDX_WORDS + w];
         const unsigned char* cbbase = smem + (s & 1) * SLICE_LDS;
 #pragma unroll
         for (int w = 0; w < IDX_WORDS; ++w) {
-            uint32_t word = idx_cur[w];
-            // ascending codebook order; partial unroll keeps the loads in flight within the VGPR budget
-#pragma unroll 4
-            for (int h = 0; h < per_word; ++h) {
-                const uint32_t r = word & ((1u << IDX_BITS) - 1);
-                word >>= IDX_BITS;
-                const unsigned char* row = cbbase + r * PITCH;
-                cbbase += CB_BYTES;
+            uint32_t word[TPL];
 #pragma unroll
-                for (int c = 0; c < Q; ++c) {
-                    const float4 vv = *reinterpret_cast<const float4*>(row + c * 16);
-                    acc[4 * c + 0] = __fadd_rn(acc[4 * c + 0], vv.x);
-                    acc[4 * c + 1] = __fadd_rn(acc[4 * c + 1], vv.y);
-                    acc[4 * c + 2] = __fadd_rn(acc[4 * c + 2], vv.z);
-                    acc[4 * c + 3] = __fadd_rn(acc[4 * c + 3], vv.w);
+            for (int t = 0; t < TPL; ++t) word[t] = idx_cur[t][w];
+            // ascending codebook order; partial unroll keeps the loads in flight within the VGPR budget
+#pragma unroll(TPL == 1 ? 4 : 2)
+            for (int h = 0; h < per_word; ++h) {
+#pragma unroll
+                for (int t = 0; t < TPL; ++t) {
+                    const uint32_t r = word[t] & ((1u << IDX_BITS) - 1);
+                    word[t] >>= IDX_BITS;
+                    const unsigned char* row = cbbase + r * PITCH;
+#pragma unroll
+                    for (int c = 0; c < Q; ++c) {
+                        const float4 vv = *reinterpret_cast<const float4*>(row + c * 16);
+                        acc[t][4 * c + 0] = __fadd_rn(acc[t][4 * c + 0], vv.x);
+                        acc[t][4 * c + 1] = __fadd_rn(acc[t][4 * c + 1], vv.y);
+                        acc[t][4 * c + 2] = __fadd_rn(acc[t][4 * c + 2], vv.z);
+                        acc[t][4 * c + 3] = __fadd_rn(acc[t][4 * c + 3], vv.w);
+                    }
                 }
+                cbbase += CB_BYTES;
                 if constexpr (GROUPED) {
                     // codebooks past CB are padding (zero rows) and belong to no group
                     if (cb < CB && (++in_group == group || cb + 1 == CB)) {
                         const float sc = scales[gi];
 #pragma unroll
-                        for (int i = 0; i < FB; ++i) {
-                            tot[i] = __fadd_rn(tot[i], __fmul_rn(acc[i], sc));
-                            acc[i] = 0.0f;
-                        }
+                        for (int t = 0; t < TPL; ++t)
+#pragma unroll
+                            for (int i = 0; i < FB; ++i) {
+                                tot[t][i] = __fadd_rn(tot[t][i], __fmul_rn(acc[t][i], sc));
+                                acc[t][i] = 0.0f;
+                            }
                         ++gi;
                         in_group = 0;
                     }
@@ -1011,17 +1031,32 @@ __global__ __launch_bounds__(GF_THREADS) void gather_f32_kernel(const uint8_t* _
         }
         PIMDL_COMMIT_SLICE((s + 1) & 1)
 #pragma unroll
-        for (int w = 0; w < IDX_WORDS; ++w) idx_cur[w] = idx_nxt[w];
+        for (int t = 0; t < TPL; ++t)
+#pragma unroll
+            for (int w = 0; w < IDX_WORDS; ++w) idx_cur[t][w] = idx_nxt[t][w];
         __syncthreads();
     }
 #undef PIMDL_FETCH_SLICE
 #undef PIMDL_COMMIT_SLICE
 
-    if (tok < N) {
+    const bool vec_store = (M % 4 == 0);  // then every 4-column piece is whole and 16-byte aligned
 #pragma unroll
-        for (int i = 0; i < FB; ++i) {
-            const uint32_t f = colblk * FB + i;
-            if (f < M) out[(size_t)tok * M + f] = activate(__fadd_rn(GROUPED ? tot[i] : acc[i], bias ? bias[f] : 0.0f), act);
+    for (int t = 0; t < TPL; ++t) {
+        if (tok[t] >= N) continue;
+#pragma unroll
+        for (int c = 0; c < Q; ++c) {
+            const uint32_t f = colblk * FB + 4 * c;
+            float o[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                o[e] = activate(__fadd_rn(GROUPED ? tot[t][4 * c + e] : acc[t][4 * c + e], (bias && f + e < M) ? bias[f + e] : 0.0f), act);
+            if (vec_store) {
+                if (f < M) *reinterpret_cast<float4*>(out + (size_t)tok[t] * M + f) = make_float4(o[0], o[1], o[2], o[3]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (f + e < M) out[(size_t)tok[t] * M + f + e] = o[e];
+            }
         }
     }
 }
@@ -1054,11 +1089,11 @@ int launch_i8(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_
     return hip_check(ctx, hipGetLastError(), "gather_i8_kernel launch");
 }
 
-template <int C_T, int Q, int GS, int IDX_BITS, bool GROUPED>
+template <int C_T, int Q, int GS, int IDX_BITS, bool GROUPED, int TPL>
 int launch_f32_impl(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, uint32_t n)
 {
     constexpr int LDS = 2 * GS * C_T * (16 * Q + 16);
-    auto kern = gather_f32_kernel<C_T, Q, GS, IDX_BITS, GROUPED>;
+    auto kern = gather_f32_kernel<C_T, Q, GS, IDX_BITS, GROUPED, TPL>;
     static bool attr_set = false;
     if (!attr_set) {
         int rc = hip_check(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -1067,7 +1102,7 @@ int launch_f32_impl(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, 
         if (rc) return rc;
         attr_set = true;
     }
-    dim3 grid((n + GF_THREADS - 1) / GF_THREADS, a.g.M_pad / (4 * Q));
+    dim3 grid((n + GF_THREADS * TPL - 1) / (GF_THREADS * TPL), a.g.M_pad / (4 * Q));
     hipLaunchKernelGGL(kern, grid, dim3(GF_THREADS), LDS, ctx->stream, d_idx,
                        reinterpret_cast<const float*>(a.d_lut), d_out, n, a.g.M, a.g.CB_pad, a.g.idx_row_bytes,
                        a.d_bias, a.d_scales, a.g.CB, a.desc.scale_group, a.desc.activation);
@@ -1077,8 +1112,15 @@ int launch_f32_impl(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, 
 template <int C_T, int Q, int GS, int IDX_BITS>
 int launch_f32(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, uint32_t n)
 {
-    return a.grouped ? launch_f32_impl<C_T, Q, GS, IDX_BITS, true>(ctx, a, d_idx, d_out, n)
-                     : launch_f32_impl<C_T, Q, GS, IDX_BITS, false>(ctx, a, d_idx, d_out, n);
+    // two tokens per lane halve the table traffic from L2; for batches that still give every CU two
+    // workgroups
+    const uint64_t wgs2 = (uint64_t)((n + 2 * GF_THREADS - 1) / (2 * GF_THREADS)) * (a.g.M_pad / (4 * Q));
+    const bool two = wgs2 >= 2ull * ctx->prop.multiProcessorCount;
+    if (a.grouped)
+        return two ? launch_f32_impl<C_T, Q, GS, IDX_BITS, true, 2>(ctx, a, d_idx, d_out, n)
+                   : launch_f32_impl<C_T, Q, GS, IDX_BITS, true, 1>(ctx, a, d_idx, d_out, n);
+    return two ? launch_f32_impl<C_T, Q, GS, IDX_BITS, false, 2>(ctx, a, d_idx, d_out, n)
+               : launch_f32_impl<C_T, Q, GS, IDX_BITS, false, 1>(ctx, a, d_idx, d_out, n);
 }
 
 }  // namespace

@@ -245,6 +245,24 @@ def test_scale_per_codebook_group(ctx, group, C, v, CB, M):
     amm.close()
 
 
+@pytest.mark.parametrize("kind", ["f32", "grouped"])
+def test_two_tokens_per_lane_in_the_fp32_table_gather(ctx, kind):
+    """Wide outputs make the fp32-table gather give each lane two tokens (rows t and t + 256 of a 512-token
+    block); the last block is ragged in both halves' sense: 1100 = 2 * 512 + 76."""
+    N, v, CB, C, M = 1100, 4, 8, 16, 2752
+    x, cent, lut, bias = make_case(77, N, CB * v, v, C, M, "f32" if kind == "f32" else "i8")
+    want_idx = oracle.index_calculation(x, cent, v, threads=THREADS)
+    if kind == "f32":
+        amm = ctx.amm(cent, lut, None, bias, max_n=N)
+        np.testing.assert_allclose(amm.run(x), oracle.gather_f32(want_idx, lut, bias, threads=THREADS), rtol=1e-5, atol=1e-6)
+    else:
+        scales = np.random.default_rng(3).uniform(1e-3, 0.1, 3).astype(np.float32)
+        amm = ctx.amm(cent, lut, scales, bias, max_n=N, scale_group=3)
+        want = oracle.gather_i8_grouped(want_idx, lut, scales, bias, 3, threads=THREADS)
+        assert np.array_equal(amm.run(x).view(np.uint32), want.view(np.uint32))
+    amm.close()
+
+
 def test_scale_groups_from_lutgen(ctx):
     """lutgen with per-group quantisation -> operator with the same grouping: closer to the fp32 product
     than the per-tensor quantisation of the same table, and equal to the oracle on the generated table."""
