@@ -498,11 +498,15 @@ constexpr int oh_tok_item(int tm) { return OH_WAVES * tm * 16; }
 constexpr int oh_slice_cbs(int) { return 16; }
 // LUT slice buffers in LDS (prefetch distance = buffers - 1); two workgroups must fit in a CU's LDS
 constexpr int oh_nbuf(int) { return 3; }
+// Up to 8 centroids ("paired"): two codebooks share the 16 K-slots of a lane, so a slice entry is a pair of
+// codebooks, its index is the whole byte (one nibble per codebook) and the table holds two-hot vectors.
+constexpr int oh_table_bytes(bool p8) { return p8 ? 4096 : 256; }
+constexpr int oh_iwords(int tn, bool p8) { return p8 ? oh_slice_cbs(tn) / 4 : oh_slice_cbs(tn) / 8; }
 // one-hot table + LUT slice buffers + index buffers
-constexpr int oh_lds_bytes(int tn)
+constexpr int oh_lds_bytes(int tn, bool p8 = false)
 {
     // (every wave keeps the index words of a whole 64-token block, whatever part of it it owns)
-    return 256 + oh_nbuf(tn) * oh_slice_cbs(tn) * 16 * tn * 16 + oh_nbuf(tn) * OH_WAVES * 64 * (oh_slice_cbs(tn) / 2);
+    return oh_table_bytes(p8) + oh_nbuf(tn) * oh_slice_cbs(tn) * 16 * tn * 16 + oh_nbuf(tn) * OH_WAVES * 64 * 4 * oh_iwords(tn, p8);
 }
 
 // Loads through the scalar data cache (read only) of wave-uniform addresses; they count on the
@@ -538,7 +542,7 @@ __device__ __forceinline__ void oh_wait(v4i (&a)[TN], v4i (&b)[TM])
 // can only issue an MFMA every ~30 cycles; two keep the matrix core at its ~21).  Smaller wave
 // tiles with more waves were slower: a K-step must hold enough MFMAs (TM*TN) to cover the LDS
 // latency of the next K-step's operands.
-template <int TN, int TM>
+template <int TN, int TM, bool P8>
 __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
     const uint8_t* __restrict__ idx, const int8_t* __restrict__ lut, float* __restrict__ out,
     int32_t* __restrict__ acc_out, uint32_t N, uint32_t M, uint32_t CB_pad, uint32_t idx_row_bytes,
@@ -550,7 +554,7 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
     constexpr int G = oh_slice_cbs(TN);            // codebooks per slice
     constexpr int SLICE = G * WN * 16;             // bytes of one codebook slice
     constexpr int KSTEPS = G / 4;
-    constexpr int IWORDS = G / 8;                  // 32-bit index words per token and slice
+    constexpr int IWORDS = oh_iwords(TN, P8);      // 32-bit index words per token and slice
     constexpr int NBLK = SLICE / 1024;             // 1 KB blocks (one copy instruction of a wave) per slice
     constexpr int DMA_PER_WAVE = (NBLK + OH_WAVES - 1) / OH_WAVES;
 
@@ -559,10 +563,10 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     constexpr int NBUF = oh_nbuf(TN), NIBUF = NBUF;
     constexpr int PD = NBUF - 1;  // prefetch distance of the LUT stream, in slices
-    constexpr uint32_t BUF0 = 256;  // the table sits at LDS offset 0: entry address = nibble * 16
+    constexpr uint32_t BUF0 = oh_table_bytes(P8);  // the table sits at LDS offset 0: entry address = nibble (byte) * 16
     constexpr uint32_t IBUF0 = BUF0 + NBUF * SLICE;
-    constexpr uint32_t IBYTES = OH_WAVES * 64 * (G / 2);      // index bytes of one slice (a 64-token block per wave)
-    constexpr uint32_t IWAVE = 64 * (G / 2);                  // ... of one wave's 64 tokens
+    constexpr uint32_t IBYTES = OH_WAVES * 64 * 4 * IWORDS;   // index bytes of one slice (a 64-token block per wave)
+    constexpr uint32_t IWAVE = 64 * 4 * IWORDS;               // ... of one wave's 64 tokens
     constexpr int IX_OPS = IWORDS;                            // 64 lanes x 4 B = 64 tokens x 1 word
     constexpr int DMA_OPS = DMA_PER_WAVE + IX_OPS;            // memory operations per wave and slice
 
@@ -575,7 +579,18 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
     const uint32_t my_items = (n_items - blockIdx.x + gridDim.x - 1) / gridDim.x;
     const uint32_t total = my_items * nslices;
 
-    if (threadIdx.x < 64) {  // entry e = 16 bytes, byte e is 1
+    if constexpr (P8) {
+        // entry e (index byte: codebook 2k in the low nibble, 2k+1 in the high one) = 16 bytes with byte
+        // (e & 15) and byte 8 + (e >> 4) set; a nibble of 8 or more (no such centroid) sets nothing
+        static_assert(OH_THREADS == 256, "one table entry per thread");
+        const uint32_t lo = threadIdx.x & 15, hi = threadIdx.x >> 4;
+        uint32_t w[4];
+#pragma unroll
+        for (uint32_t q = 0; q < 4; ++q)
+            w[q] = ((lo < 8 && (lo >> 2) == q) ? (1u << (8 * (lo & 3))) : 0u) |
+                   ((hi < 8 && 2 + (hi >> 2) == q) ? (1u << (8 * (hi & 3))) : 0u);
+        reinterpret_cast<uint4*>(smem)[threadIdx.x] = make_uint4(w[0], w[1], w[2], w[3]);
+    } else if (threadIdx.x < 64) {  // entry e = 16 bytes, byte e is 1
         const uint32_t e = threadIdx.x >> 2, w = threadIdx.x & 3;
         reinterpret_cast<uint32_t*>(smem)[threadIdx.x] = ((e >> 2) == w) ? (1u << (8 * (e & 3))) : 0u;
     }
@@ -643,7 +658,7 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
                                          (__attribute__((address_space(3))) void*)(smem + dst + 256 * i), 4, 0, 0);
     };
     auto ix_advance = [&]() {
-        ix_base += (G / 8) * 256;
+        ix_base += IWORDS * 256;
         if (++ix_s == nslices) {
             ix_s = 0;
             ix_item += gridDim.x;
@@ -659,6 +674,7 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
     // after masking, one v_bfe_u32 yields nibble * 16: the byte offset of the one-hot table entry.
     const uint32_t pre_shift = (g & 1) ? 0u : 4u;
     const uint32_t byte_shift = 8 * (g >> 1);
+    const uint32_t rot8 = (8 * g + 28) & 31;  // rotate right by 8g - 4
     const uint32_t ix_lane = IBUF0 + wave * IWAVE + (((wave * (TM * 16)) & 63) + j) * 4;
     // The index words are read with inline assembly: the compiler cannot tell these reads from the
     // LDS ranges the copy operations in flight are writing, and would wait for all of them first.
@@ -678,7 +694,12 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
 #pragma unroll
         for (int t = 0; t < TM; ++t)
 #pragma unroll
-            for (int i = 0; i < IWORDS; ++i) iwm[t][i] = (raw[t][i] << pre_shift) & 0xF0F0F0F0u;
+            for (int i = 0; i < IWORDS; ++i) {
+                // paired: word i belongs to K-step i and this lane's pair is byte g of it; rotating that
+                // byte to bits 4..11 leaves byte * 16, the table entry's offset
+                if constexpr (P8) iwm[t][i] = __builtin_amdgcn_alignbit(raw[t][i], raw[t][i], rot8) & 0xFF0u;
+                else iwm[t][i] = (raw[t][i] << pre_shift) & 0xF0F0F0F0u;
+            }
     };
 
     v4i acc[TM][TN];
@@ -817,7 +838,7 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
             });
 #pragma unroll
             for (int t = 0; t < TM; ++t) {
-                const uint32_t entry = __builtin_amdgcn_ubfe(iwm[t][ks / 2], 16 * (ks & 1) + byte_shift, 8);
+                const uint32_t entry = P8 ? iwm[t][ks] : __builtin_amdgcn_ubfe(iwm[t][ks / 2], 16 * (ks & 1) + byte_shift, 8);
                 lds_read<0>(b_op[ks & 1][t], entry);
             }
         };
@@ -854,13 +875,14 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
     }
 }
 
-template <int TN, int TM>
+template <int TN, int TM, bool P8>
 int launch_onehot_tm(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_t* d_acc, uint32_t n,
                      const Epilogue& ep)
 {
-    constexpr int LDS = oh_lds_bytes(TN);
+    constexpr int LDS = oh_lds_bytes(TN, P8);
+    static_assert(2 * LDS <= 160 * 1024, "two workgroups per CU");
     constexpr int OH_TOK_ITEM = oh_tok_item(TM);
-    auto kern = gather_onehot_kernel<TN, TM>;
+    auto kern = gather_onehot_kernel<TN, TM, P8>;
     static bool attr_set = false;
     if (!attr_set) {
         int rc = hip_check(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -873,23 +895,24 @@ int launch_onehot_tm(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out,
     const uint32_t n_items = n_token_tiles * (a.g.M_pad / (16 * TN));
     uint32_t grid = ctx->prop.multiProcessorCount * 2;  // two workgroups per CU, see plan_geometry
     if (grid > n_items) grid = n_items;
+    const uint32_t slice_entries = P8 ? a.g.CB_pad / 2 : a.g.CB_pad;  // codebooks, or pairs of them
     const XcdMap xmap = choose_xcd_map(a.g.M_pad / (16 * TN), n_token_tiles, grid,
-                                       (uint64_t)a.g.CB_pad * 16 * a.g.M_pad, (uint64_t)n * a.g.idx_row_bytes);
+                                       (uint64_t)slice_entries * 16 * a.g.M_pad, (uint64_t)n * a.g.idx_row_bytes);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(OH_THREADS), LDS, ctx->stream, d_idx,
-                       reinterpret_cast<const int8_t*>(a.d_lut), d_out, d_acc, n, a.g.M, a.g.CB_pad,
+                       reinterpret_cast<const int8_t*>(a.d_lut), d_out, d_acc, n, a.g.M, slice_entries,
                        a.g.idx_row_bytes, n_token_tiles, n_items, ep, xmap);
     return hip_check(ctx, hipGetLastError(), "gather_onehot_kernel launch");
 }
 
 // 256-token items (TM = 4) need fewer LDS reads and copies per MFMA; when the batch does not offer
 // two of them per CU, 128-token items (TM = 2) put a second wave on every SIMD instead.
-template <int TN>
+template <int TN, bool P8>
 int launch_onehot(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_t* d_acc, uint32_t n,
                   const Epilogue& ep)
 {
     const uint64_t items4 = (uint64_t)((n + oh_tok_item(4) - 1) / oh_tok_item(4)) * (a.g.M_pad / (16 * TN));
-    if (items4 < 2ull * ctx->prop.multiProcessorCount) return launch_onehot_tm<TN, 2>(ctx, a, d_idx, d_out, d_acc, n, ep);
-    return launch_onehot_tm<TN, 4>(ctx, a, d_idx, d_out, d_acc, n, ep);
+    if (items4 < 2ull * ctx->prop.multiProcessorCount) return launch_onehot_tm<TN, 2, P8>(ctx, a, d_idx, d_out, d_acc, n, ep);
+    return launch_onehot_tm<TN, 4, P8>(ctx, a, d_idx, d_out, d_acc, n, ep);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1169,15 +1192,20 @@ bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::s
         // One-hot matrix-core kernel: an item is 256 tokens x 16*TN columns, all items cost the
         // same.  Take the TN that fills the persistent grid (two workgroups per CU) most evenly for
         // the largest batch this operator will see; among equals the widest (fewest LDS reads).
-        g->C_tile = 16;
+        // up to 8 centroids: two codebooks share a lane's 16 K-slots (C_tile 8); 96-column tiles then do not
+        // leave room for two workgroups per CU
+        const bool paired = C <= 8;
+        g->C_tile = paired ? 8 : 16;
         const uint32_t slots = 2 * (num_cus ? num_cus : 256);
         const uint32_t tiles = (d.max_n + 255) / 256;
         double best = -1.0;
-        if (col_block_hint && col_block_hint != 96 && col_block_hint != 64 && col_block_hint != 48) {
-            *why = "column tile hint must be 48, 64 or 96 for this operator";
+        if (col_block_hint && col_block_hint != 64 && col_block_hint != 48 && (paired || col_block_hint != 96)) {
+            *why = paired ? "column tile hint must be 48 or 64 for this operator"
+                          : "column tile hint must be 48, 64 or 96 for this operator";
             return false;
         }
         for (uint32_t tn : {6u, 4u, 3u}) {
+            if (paired && tn == 6) continue;
             if (col_block_hint && col_block_hint != 16 * tn) continue;
             const uint32_t blocks = (M + 16 * tn - 1) / (16 * tn);
             const uint64_t items = (uint64_t)tiles * blocks;
@@ -1194,7 +1222,7 @@ bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::s
         g->gather_threads = 256;
         g->tokens_per_wg = 256;
         g->row_pitch = 16;
-        g->gather_lds_bytes = 256 + 3 * (g->cb_per_slice * g->col_block * 16 + 256 * (g->cb_per_slice / 2));
+        g->gather_lds_bytes = (uint32_t)oh_lds_bytes((int)g->q, paired);
         g->M_pad = (M + g->col_block - 1) / g->col_block * g->col_block;
         g->ccs_cb_per_wg = ccs_cb_per_wg(v);
         g->ccs_row_floats = g->ccs_cb_per_wg * v;
@@ -1257,10 +1285,17 @@ int launch_gather(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, in
         ep.bias = a.d_bias;
         ep.act = a.desc.activation;
         if (g.gather_kind == 1) {
-            switch (g.q) {
-                case 3: return launch_onehot<3>(ctx, a, d_idx, d_out, d_acc, n, ep);
-                case 4: return launch_onehot<4>(ctx, a, d_idx, d_out, d_acc, n, ep);
-                case 6: return launch_onehot<6>(ctx, a, d_idx, d_out, d_acc, n, ep);
+            if (g.C_tile == 8) {
+                switch (g.q) {
+                    case 3: return launch_onehot<3, true>(ctx, a, d_idx, d_out, d_acc, n, ep);
+                    case 4: return launch_onehot<4, true>(ctx, a, d_idx, d_out, d_acc, n, ep);
+                }
+            } else {
+                switch (g.q) {
+                    case 3: return launch_onehot<3, false>(ctx, a, d_idx, d_out, d_acc, n, ep);
+                    case 4: return launch_onehot<4, false>(ctx, a, d_idx, d_out, d_acc, n, ep);
+                    case 6: return launch_onehot<6, false>(ctx, a, d_idx, d_out, d_acc, n, ep);
+                }
             }
             return set_error(ctx, PIMDL_ERR_UNSUPPORTED, "no one-hot gather kernel for %u column groups", g.q);
         }

@@ -131,15 +131,19 @@ static void retile_lut(const T* lut, T* tiled, const AmmGeom& g, uint32_t row_el
             }
 }
 
-// canonical [CB][C][M] -> [M_pad/col_block][CB_pad][col_block][16], zero padded (C <= 16)
+// canonical [CB][C][M] -> [M_pad/col_block][CB_pad][col_block][16], zero padded (C <= 16);
+// C_tile 8 (C <= 8): [M_pad/col_block][CB_pad/2][col_block][2][8], codebooks 2k and 2k+1 side by side
 static void retile_lut_onehot(const int8_t* lut, int8_t* tiled, const AmmGeom& g)
 {
     const uint32_t wn = g.col_block;
+    const bool paired = g.C_tile == 8;
     for (uint32_t cb = 0; cb < g.CB; ++cb)
         for (uint32_t c = 0; c < g.C; ++c) {
             const int8_t* src = lut + ((size_t)cb * g.C + c) * g.M;
+            const uint32_t entry = paired ? cb / 2 : cb, entries = paired ? g.CB_pad / 2 : g.CB_pad;
+            const uint32_t slot = paired ? 8 * (cb & 1) + c : c;
             for (uint32_t f = 0; f < g.M; ++f)
-                tiled[((((size_t)(f / wn) * g.CB_pad + cb) * wn) + f % wn) * 16 + c] = src[f];
+                tiled[((((size_t)(f / wn) * entries + entry) * wn) + f % wn) * 16 + slot] = src[f];
         }
 }
 

@@ -29,8 +29,9 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_struct_layouts_match_the_header():
-    # pimdl_amm_desc: 8 x uint32 + float; pimdl_amm_timing: 3 floats
-    assert ctypes.sizeof(pimdl.AmmDesc) == 36
+    # pimdl_amm_desc: 8 x uint32 + float + uint32 (activation); pimdl_amm_timing: 3 floats
+    assert ctypes.sizeof(pimdl.AmmDesc) == 40
+    assert pimdl.AmmDesc.activation.offset == 36
     assert ctypes.sizeof(pimdl.AmmTiming) == 12
     assert ctypes.sizeof(pimdl.AmmGeometry) == 14 * 4
     assert ctypes.sizeof(pimdl.DeviceInfo) == 64 + 32 + 4 * 3 + 4 + 8  # 4 bytes of padding before the u64

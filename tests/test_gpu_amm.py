@@ -190,9 +190,11 @@ def test_near_ties_follow_the_scan_not_the_true_argmin(ctx):
     amm.close()
 
 
-def test_gather_from_given_indices_and_invariants(ctx):
+@pytest.mark.parametrize("C", [16, 8, 5])
+def test_gather_from_given_indices_and_invariants(ctx, C):
+    """C <= 8 runs the paired form of the matrix-core gather (two codebooks per index byte, odd CB)."""
     rng = np.random.default_rng(21)
-    N, CB, C, M, v = 300, 40, 16, 192, 4
+    N, CB, M, v = 300, 41 if C < 16 else 40, 192, 4
     cent = rng.standard_normal((CB, C, v)).astype(np.float32)
     lut = rng.integers(-128, 128, (CB, C, M)).astype(np.int8)
     idx = rng.integers(0, C, (N, CB)).astype(np.uint16)
