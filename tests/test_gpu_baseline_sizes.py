@@ -75,3 +75,9 @@ def test_vit_base_sweep_full_batch(env, v, C, lut_kind):
 @pytest.mark.parametrize("v,C", [(2, 16), (4, 16), (8, 32)])
 def test_vit_base_ffn2_full_batch(env, v, C):
     run_and_check_sample(env[1], 29 + v, 12608, 3072, v, C, 768, "i8", sample=96)
+
+
+def test_reference_single_amm_search_space_shape(env):
+    """The shape of the reference's 89 single-AMM tuning configs: N = 32768, 1024 -> 4096, 256 codebooks of
+    16 centroids (512 MB of fp32 output, 128 token tiles x 64 column tiles)."""
+    run_and_check_sample(env[1], 41, 32768, 1024, 4, 16, 4096, "i8", sample=64)
