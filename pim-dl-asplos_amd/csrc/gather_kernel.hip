@@ -116,10 +116,14 @@ __device__ __forceinline__ float activate(float y, uint32_t act)  // act is unif
     return act == PIMDL_ACT_GELU_TANH ? gelu_tanh(y) : y;
 }
 
+// ACT: the epilogues are compiled once per activation and chosen by a (uniform) branch; as a select the
+// activation's arithmetic would run for every element of every launch
+template <bool ACT>
 __device__ __forceinline__ float dequant(int32_t acc, const Epilogue& ep, float b)
 {
     // ((float)acc * scale + lut_bias_term) + bias[f]   -- three separately rounded fp32 operations
-    return activate(__fadd_rn(__fadd_rn(__fmul_rn((float)acc, ep.scale), ep.lut_bias_term), b), ep.act);
+    const float y = __fadd_rn(__fadd_rn(__fmul_rn((float)acc, ep.scale), ep.lut_bias_term), b);
+    return ACT ? gelu_tanh(y) : y;
 }
 
 template <int I, int N, class F>
@@ -323,7 +327,10 @@ __global__ __launch_bounds__(GATHER_THREADS, 4) void gather_i8_kernel(
     // 4*g .. 4*g+3 of every 16-column chunk for token j.  It runs right after a top-of-slice wait, so
     // its stores have a whole slice to drain before anything waits on the memory counter again; the
     // bias values are fetched first so that no store sits between a load and its use.
-    auto epilogue = [&](uint32_t item) {
+    // (always_inline: called from two places; as a real function it would take the accumulators, and
+    // registers whose loads are still in flight, through memory)
+    auto epilogue_as = [&](uint32_t item, auto actc) __attribute__((always_inline)) {
+        constexpr bool ACT = decltype(actc)::value;
         const uint32_t colblk = item / n_token_tiles;
         const uint32_t tok0 = (item % n_token_tiles) * TOK_ITEM + wave * (TG * 16);
         const bool vec_store = (M % 4 == 0);
@@ -353,10 +360,10 @@ __global__ __launch_bounds__(GATHER_THREADS, 4) void gather_i8_kernel(
                 acc[t][c] = (v4i){0, 0, 0, 0};
                 if (tok >= N || f >= M) continue;
                 float4 o;
-                o.x = dequant(a[0], ep, bv[c].x);
-                o.y = dequant(a[1], ep, bv[c].y);
-                o.z = dequant(a[2], ep, bv[c].z);
-                o.w = dequant(a[3], ep, bv[c].w);
+                o.x = dequant<ACT>(a[0], ep, bv[c].x);
+                o.y = dequant<ACT>(a[1], ep, bv[c].y);
+                o.z = dequant<ACT>(a[2], ep, bv[c].z);
+                o.w = dequant<ACT>(a[3], ep, bv[c].w);
                 if (vec_store) {  // M % 4 == 0 and f % 4 == 0: the whole float4 is in range and aligned
                     *reinterpret_cast<float4*>(out + (size_t)tok * M + f) = o;
                     if (acc_out) *reinterpret_cast<v4i*>(acc_out + (size_t)tok * M + f) = a;
@@ -372,6 +379,10 @@ __global__ __launch_bounds__(GATHER_THREADS, 4) void gather_i8_kernel(
                 }
             }
         }
+    };
+    auto epilogue = [&](uint32_t item) __attribute__((always_inline)) {
+        if (ep.act == PIMDL_ACT_GELU_TANH) epilogue_as(item, std::true_type{});
+        else epilogue_as(item, std::false_type{});
     };
 
     for (uint32_t k = 0; k < total; ++k) {
@@ -713,7 +724,8 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
     // use, i.e. for every output store issued so far and for the slices being prefetched, once per
     // group of stores.  With scalar loads the epilogue contains no such wait and its stores leave
     // back to back.
-    auto epilogue = [&](uint32_t item) -> bool {
+    auto epilogue_as = [&](uint32_t item, auto actc) __attribute__((always_inline)) -> bool {
+        constexpr bool ACT = decltype(actc)::value;
         // j and g pass through an opaque asm so that none of the address arithmetic below is
         // loop-invariant for the compiler: hoisted out of the slice loop it would occupy dozens of
         // registers for the whole kernel
@@ -746,10 +758,10 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
                 const v4i a = acc[t][c];
                 acc[t][c] = (v4i){0, 0, 0, 0};
                 float4 o;
-                o.x = dequant(a[0], ep, bv.x);
-                o.y = dequant(a[1], ep, bv.y);
-                o.z = dequant(a[2], ep, bv.z);
-                o.w = dequant(a[3], ep, bv.w);
+                o.x = dequant<ACT>(a[0], ep, bv.x);
+                o.y = dequant<ACT>(a[1], ep, bv.y);
+                o.z = dequant<ACT>(a[2], ep, bv.z);
+                o.w = dequant<ACT>(a[3], ep, bv.w);
                 if (full) {  // workgroup-uniform: every token and column of the tile exists
                     // streaming store: the output is not read again by this kernel
                     typedef float v4f __attribute__((ext_vector_type(4)));
@@ -773,6 +785,9 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
             }
         }
         return full;
+    };
+    auto epilogue = [&](uint32_t item) __attribute__((always_inline)) -> bool {
+        return ep.act == PIMDL_ACT_GELU_TANH ? epilogue_as(item, std::true_type{}) : epilogue_as(item, std::false_type{});
     };
 
     // ---- prologue: slices 0 .. PD-1, index words 0 .. PD ------------------------------------------
