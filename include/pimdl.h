@@ -86,6 +86,8 @@ typedef struct pimdl_amm_desc {
     uint32_t activation;        /* pimdl_activation */
 } pimdl_amm_desc;
 
+typedef struct pimdl_amm_group pimdl_amm_group; /* operators that read the same input rows */
+
 /* Timing of the last profiled run, milliseconds on the device (HIP events on the context's
  * stream, averaged over `iters` launches of each kernel on its own). */
 typedef struct pimdl_amm_timing {
@@ -144,6 +146,20 @@ PIMDL_API int pimdl_amm_run(pimdl_amm* amm, const float* in, uint32_t n, float* 
  * Always synchronous. */
 PIMDL_API int pimdl_amm_run_debug(pimdl_amm* amm, const float* in, uint32_t n, float* out,
                                   uint16_t* idx_out, int32_t* acc_out);
+
+/* Operators that read the same rows: the reference's layer calls amm_host three times on one input for
+ * the separate Q, K and V projections (src/host/transformer_layer.cpp:335-343), searching the same
+ * activations against three sets of centroids.  A group searches the codebooks of all its operators
+ * in ONE launch (the input is read once and the launch's fixed cost is paid once), then runs each
+ * operator's gather; results are bit for bit those of pimdl_amm_run on each operator.
+ *   Conditions: same context, input_feature_len, sub_vec_len (2, 4 or 8) and num_centroid (<= 32), the same
+ *   LUT type, num_codebook a multiple of 32; otherwise PIMDL_ERR_UNSUPPORTED / PIMDL_ERR_INVALID and the
+ *   caller runs the operators one by one.  The group borrows its operators: destroy it before them.
+ *   outs[i]: fp32 [n][M_i] of operator i, host or device; n <= the smallest max_n. */
+PIMDL_API int pimdl_amm_group_create(pimdl_ctx* ctx, pimdl_amm* const* amms, uint32_t count,
+                                     pimdl_amm_group** out);
+PIMDL_API int pimdl_amm_group_run(pimdl_amm_group* group, const float* in, uint32_t n, float* const* outs);
+PIMDL_API int pimdl_amm_group_destroy(pimdl_amm_group* group);
 
 /* Runs the two kernels `iters` times each on device-resident buffers and reports the average
  * device time of each.  in/out must be DEVICE pointers. */

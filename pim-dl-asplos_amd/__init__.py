@@ -30,7 +30,7 @@ EXPORTS = ["pimdl_init", "pimdl_destroy", "pimdl_last_error", "pimdl_set_stream"
            "pimdl_amm_profile", "pimdl_index_calculation", "pimdl_amm_index_calculation", "pimdl_lut_gather",
            "pimdl_amm_run_tiled", "pimdl_lut_gather_tiled", "pimdl_lutgen",
            "pimdl_layer_norm", "pimdl_get_device_info", "pimdl_amm_get_geometry", "pimdl_diag_bandwidth",
-           "pimdl_diag_mfma_error"]
+           "pimdl_diag_mfma_error", "pimdl_amm_group_create", "pimdl_amm_group_run", "pimdl_amm_group_destroy"]
 
 
 class PimdlError(RuntimeError):
@@ -128,6 +128,9 @@ def lib():
     L.pimdl_amm_get_geometry.argtypes = [vp, ctypes.POINTER(AmmGeometry)]
     L.pimdl_diag_bandwidth.argtypes = [vp, u64, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float)]
     L.pimdl_diag_mfma_error.argtypes = [vp, ctypes.c_uint32, ctypes.POINTER(ctypes.c_float)]
+    L.pimdl_amm_group_create.argtypes = [vp, ctypes.POINTER(vp), u32, ctypes.POINTER(vp)]
+    L.pimdl_amm_group_run.argtypes = [vp, vp, u32, ctypes.POINTER(vp)]
+    L.pimdl_amm_group_destroy.argtypes = [vp]
     for name in EXPORTS:
         if name != "pimdl_last_error":
             getattr(L, name).restype = ctypes.c_int
@@ -240,11 +243,44 @@ class Context:
                                            ctypes.c_float(eps)))
         return y
 
+    def amm_group(self, amms):
+        return AmmGroup(self, amms)
+
     def amm(self, centroids, lut, scales=None, bias=None, max_n=8192, lut_bias=0.0, bias_mode=BIAS_ONCE,
             scale_group=0, col_block=0, activation=ACT_NONE):
         """col_block: width of the gather kernel's column tile (0 = chosen by the library).
         activation: ACT_GELU_TANH applies the tanh form of GELU to the output inside the gather's epilogue."""
         return Amm(self, centroids, lut, scales, bias, max_n, lut_bias, bias_mode, scale_group, col_block, activation)
+
+
+class AmmGroup:
+    """Operators of one context that read the same input rows (separate Q/K/V projections): one search launch
+    over all their codebooks, then each operator's gather.  Raises PimdlError (UNSUPPORTED / INVALID) when the
+    operators cannot share a search; run them one by one then."""
+
+    def __init__(self, ctx, amms):
+        self.ctx, self.amms = ctx, list(amms)
+        handles = (ctypes.c_void_p * len(self.amms))(*[a._h for a in self.amms])
+        self._h = ctypes.c_void_p()
+        ctx._check(lib().pimdl_amm_group_create(ctx._h, handles, len(self.amms), ctypes.byref(self._h)))
+
+    def close(self):
+        if self._h and self.ctx._h:
+            lib().pimdl_amm_group_destroy(self._h)
+        self._h = ctypes.c_void_p()
+
+    def run(self, x):
+        x = np.ascontiguousarray(x, np.float32)
+        n = x.shape[0]
+        outs = [np.empty((n, a.M), np.float32) for a in self.amms]
+        ptrs = (ctypes.c_void_p * len(outs))(*[o.ctypes.data for o in outs])
+        self.ctx._check(lib().pimdl_amm_group_run(self._h, _ptr(x), n, ptrs))
+        return outs
+
+    def run_ptr(self, in_ptr, n, out_ptrs):
+        """Raw addresses (device or host); asynchronous for device memory."""
+        ptrs = (ctypes.c_void_p * len(out_ptrs))(*out_ptrs)
+        self.ctx._check(lib().pimdl_amm_group_run(self._h, ctypes.c_void_p(in_ptr), n, ptrs))
 
 
 class Amm:

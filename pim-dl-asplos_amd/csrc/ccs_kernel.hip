@@ -710,8 +710,10 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
                                                                  uint8_t* __restrict__ idx, uint32_t N,
                                                                  uint32_t K, uint32_t CB, uint32_t C,
                                                                  uint32_t idx_row_bytes, int idx_tiled, int vec_ok,
-                                                                 uint32_t tiles_cb, uint32_t total_tiles, uint32_t num_cus)
+                                                                 uint32_t tiles_cb, uint32_t total_tiles, uint32_t tiles_x)
 {
+    // K is the length of an activation row.  tiles_x < tiles_cb: the codebooks are those of several operators
+    // that read the same row (tiles_x codebook tiles each), so the activation columns wrap around.
     using S = CcsMfmaShape<V, WIDE>;
     constexpr int TF = S::TF, PITCH = S::PITCH, TT = S::TILE_TOKENS, CBW = S::CBW, TG = S::TG, RCB = S::RCB;
     constexpr int XSTEP = WIDE ? V : 2 * V;  // activation floats per pair
@@ -733,7 +735,7 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
     const uint32_t fr0 = threadIdx.x / F4_PER_ROW;
     auto fetch = [&](float4 (&pf)[PASSES], uint32_t tile_id) {
         const uint32_t t_tok0 = (tile_id / tiles_cb) * TT;
-        const uint32_t col = (tile_id % tiles_cb) * TF + 4 * fq;
+        const uint32_t col = ((tile_id % tiles_cb) % tiles_x) * TF + 4 * fq;
 #pragma unroll
         for (int i = 0; i < PASSES; ++i) {
             uint32_t tok = t_tok0 + fr0 + i * ROWS_PER_PASS;
@@ -760,7 +762,6 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
     // A wave's priority falls as its workgroup progresses through its share: whoever is behind goes first.
     const uint32_t my_tiles = (total_tiles - blockIdx.x + gridDim.x - 1) / gridDim.x;
     uint32_t tiles_done = 0;
-    (void)num_cus;
     for (uint32_t tile_id = blockIdx.x; tile_id < total_tiles; tile_id += gridDim.x) {
         switch (4 * tiles_done / my_tiles) {
             case 0: __builtin_amdgcn_s_setprio(3); break;
@@ -1160,7 +1161,8 @@ static bool ccs_f32_only()
 }
 
 template <int V, bool WIDE>
-int launch_ccs_bf16(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_cent, uint8_t* d_idx, uint32_t n)
+int launch_ccs_bf16(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_cent, uint8_t* d_idx, uint32_t n,
+                    uint32_t x_cols)
 {
     using S = CcsMfmaShape<V, WIDE>;
     const uint32_t tiles_cb = g.CB_pad / S::RCB;  // CB_pad is a multiple of 32
@@ -1174,7 +1176,9 @@ int launch_ccs_bf16(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d
     }
     const uint32_t slots = (uint32_t)ctx->prop.multiProcessorCount * (uint32_t)per_cu;
     dim3 grid(total < slots ? total : slots);
-    const int vec_ok = (g.K % 4 == 0) && ((reinterpret_cast<uintptr_t>(d_x) & 15) == 0);
+    const uint32_t row = x_cols ? x_cols : g.K;  // floats per activation row
+    const uint32_t tiles_x = x_cols ? x_cols / S::TF : tiles_cb;
+    const int vec_ok = (row % 4 == 0) && ((reinterpret_cast<uintptr_t>(d_x) & 15) == 0);
     const float* aux = d_cent + (size_t)g.CB * g.C * g.v;
     const float* cnmax = aux + ccs_aux_floats(g);
     const float* cnmax_pad = cnmax + g.CB + (size_t)(g.CB_pad / 2) * (g.v + 1) * 64;
@@ -1182,31 +1186,34 @@ int launch_ccs_bf16(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d
     const uint4* aux_b = reinterpret_cast<const uint4*>(bf);
     const float* cn16 = bf + ccs_bf16_units(g) * ccs_bf16_nm(V) * 64 * 4;
     hipLaunchKernelGGL((ccs_bf16_kernel<V, WIDE>), grid, dim3(CCS_THREADS), 0, ctx->stream, d_x, d_cent, aux_b, cn16, cnmax_pad,
-                       d_idx, n, g.K, g.CB, g.C, g.idx_row_bytes, (int)g.idx_tiled, vec_ok, tiles_cb, total,
-                       (uint32_t)ctx->prop.multiProcessorCount);
+                       d_idx, n, row, g.CB, g.C, g.idx_row_bytes, (int)g.idx_tiled, vec_ok, tiles_cb, total, tiles_x);
     return hip_check(ctx, hipGetLastError(), "ccs_bf16_kernel launch");
 }
 
 template <int IDX_BITS>
-int launch_ccs_bits(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_cent, uint8_t* d_idx, uint32_t n)
+int launch_ccs_bits(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_cent, uint8_t* d_idx, uint32_t n,
+                    uint32_t x_cols)
 {
     if (IDX_BITS == 8 && g.C <= 32 && !ccs_exact_only() && !ccs_f32_only()) {
         switch (g.v) {
-            case 2: return launch_ccs_bf16<2, true>(ctx, g, d_x, d_cent, d_idx, n);
-            case 4: return launch_ccs_bf16<4, true>(ctx, g, d_x, d_cent, d_idx, n);
-            case 8: return launch_ccs_bf16<8, true>(ctx, g, d_x, d_cent, d_idx, n);
+            case 2: return launch_ccs_bf16<2, true>(ctx, g, d_x, d_cent, d_idx, n, x_cols);
+            case 4: return launch_ccs_bf16<4, true>(ctx, g, d_x, d_cent, d_idx, n, x_cols);
+            case 8: return launch_ccs_bf16<8, true>(ctx, g, d_x, d_cent, d_idx, n, x_cols);
             default: break;
         }
     }
     if (IDX_BITS == 4 && !ccs_exact_only()) {
         if (!ccs_f32_only()) {
             switch (g.v) {
-                case 2: return launch_ccs_bf16<2, false>(ctx, g, d_x, d_cent, d_idx, n);
-                case 4: return launch_ccs_bf16<4, false>(ctx, g, d_x, d_cent, d_idx, n);
-                case 8: return launch_ccs_bf16<8, false>(ctx, g, d_x, d_cent, d_idx, n);
+                case 2: return launch_ccs_bf16<2, false>(ctx, g, d_x, d_cent, d_idx, n, x_cols);
+                case 4: return launch_ccs_bf16<4, false>(ctx, g, d_x, d_cent, d_idx, n, x_cols);
+                case 8: return launch_ccs_bf16<8, false>(ctx, g, d_x, d_cent, d_idx, n, x_cols);
                 default: break;
             }
         }
+    }
+    if (x_cols) return set_error(ctx, PIMDL_ERR_UNSUPPORTED, "shared-input search needs the matrix-core search kernel");
+    if (IDX_BITS == 4 && !ccs_exact_only()) {
         switch (g.v) {
             case 2: return launch_ccs_mfma<2>(ctx, g, d_x, d_cent, d_idx, n);
             case 4: return launch_ccs_mfma<4>(ctx, g, d_x, d_cent, d_idx, n);
@@ -1388,11 +1395,21 @@ uint32_t ccs_cb_per_wg(uint32_t v)
     }
 }
 
-int launch_ccs(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_cent, uint8_t* d_idx, uint32_t n)
+int launch_ccs(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_cent, uint8_t* d_idx, uint32_t n,
+               uint32_t x_cols)
 {
     if (n == 0) return PIMDL_OK;
-    return g.idx_bits == 4 ? launch_ccs_bits<4>(ctx, g, d_x, d_cent, d_idx, n)
-                           : launch_ccs_bits<8>(ctx, g, d_x, d_cent, d_idx, n);
+    return g.idx_bits == 4 ? launch_ccs_bits<4>(ctx, g, d_x, d_cent, d_idx, n, x_cols)
+                           : launch_ccs_bits<8>(ctx, g, d_x, d_cent, d_idx, n, x_cols);
+}
+
+// Can launch_ccs search the codebooks of several operators that read rows of x_cols floats?  Needs the
+// matrix-core kernel and whole codebook tiles per operator.
+bool ccs_supports_shared_input(const AmmGeom& g, uint32_t x_cols)
+{
+    if (!ccs_has_bf16(g) || ccs_exact_only() || ccs_f32_only()) return false;
+    const uint32_t tf = (ccs_bf16_wide(g) ? 8 : 16) * g.v;
+    return x_cols % tf == 0;
 }
 
 int launch_unpack_idx(Ctx* ctx, const AmmGeom& g, const uint8_t* d_idx, uint16_t* d_idx16, uint32_t n,

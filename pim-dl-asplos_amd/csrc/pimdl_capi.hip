@@ -153,6 +153,15 @@ using namespace pimdl;
 
 struct pimdl_ctx : Ctx {};
 struct pimdl_amm : Amm {};
+// Operators that read the same input rows, searched by one launch over all their codebooks.
+struct pimdl_amm_group {
+    Ctx* ctx;
+    std::vector<pimdl_amm*> members;
+    AmmGeom g;            // search geometry: the members' codebooks side by side (K = members * K of one)
+    float* d_centroids;   // the members' centroids, concatenated, + derived search data
+    uint32_t x_cols;      // floats per input row (one member's K)
+    uint32_t max_n;
+};
 
 extern "C" {
 
@@ -337,6 +346,99 @@ int pimdl_amm_destroy(pimdl_amm* a)
     (void)hipFree(a->d_scales);
     (void)hipFree(a->d_bias);
     delete a;
+    return PIMDL_OK;
+}
+
+int pimdl_amm_group_create(pimdl_ctx* ctx, pimdl_amm* const* amms, uint32_t count, pimdl_amm_group** out)
+{
+    if (!ctx) return PIMDL_ERR_INVALID;
+    if (!out) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_group_create: out is null");
+    *out = nullptr;
+    if (!amms || count < 2 || count > 16) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_group_create: 2..16 operators expected");
+    int rc = activate(ctx);
+    if (rc) return rc;
+    const Amm* first = amms[0];
+    if (!first) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_group_create: null operator");
+    uint32_t max_n = first->desc.max_n;
+    for (uint32_t i = 0; i < count; ++i) {
+        const Amm* a = amms[i];
+        if (!a) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_group_create: null operator");
+        if (a->ctx != ctx) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_group_create: operator %u belongs to another context", i);
+        if (a->g.K != first->g.K || a->g.v != first->g.v || a->g.C != first->g.C)
+            return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_group_create: operator %u differs in input_feature_len, sub_vec_len or num_centroid", i);
+        if (a->g.idx_tiled != first->g.idx_tiled || a->g.idx_bits != first->g.idx_bits)
+            return set_error(ctx, PIMDL_ERR_UNSUPPORTED, "pimdl_amm_group_create: operator %u uses another index layout (LUT type differs)", i);
+        max_n = a->desc.max_n < max_n ? a->desc.max_n : max_n;
+    }
+    if (first->g.CB != first->g.CB_pad)
+        return set_error(ctx, PIMDL_ERR_UNSUPPORTED, "pimdl_amm_group_create: num_codebook=%u is not a multiple of 32", first->g.CB);
+    AmmGeom g = first->g;
+    g.K *= count;
+    g.CB *= count;
+    g.CB_pad *= count;
+    g.idx_row_bytes *= count;
+    if (!ccs_supports_shared_input(g, first->g.K))
+        return set_error(ctx, PIMDL_ERR_UNSUPPORTED, "pimdl_amm_group_create: no shared-input search for sub_vec_len=%u, num_centroid=%u, input_feature_len=%u",
+                         g.v, g.C, first->g.K);
+    pimdl_amm_group* grp = new pimdl_amm_group();
+    grp->ctx = ctx;
+    grp->members.assign(amms, amms + count);
+    grp->g = g;
+    grp->d_centroids = nullptr;
+    grp->x_cols = first->g.K;
+    grp->max_n = max_n;
+    rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&grp->d_centroids), ccs_centroid_bytes(g)), "hipMalloc(group centroids)");
+    const size_t one = (size_t)first->g.CB * g.C * g.v;  // raw centroid floats of one member
+    for (uint32_t i = 0; i < count && !rc; ++i)
+        rc = hip_check(ctx, hipMemcpyAsync(grp->d_centroids + i * one, amms[i]->d_centroids, one * sizeof(float),
+                                           hipMemcpyDeviceToDevice, ctx->stream), "D2D centroids");
+    if (!rc) rc = launch_ccs_prep(ctx, g, grp->d_centroids);
+    if (!rc) rc = hip_check(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+    if (rc) {
+        (void)hipFree(grp->d_centroids);
+        delete grp;
+        return rc;
+    }
+    *out = grp;
+    return PIMDL_OK;
+}
+
+int pimdl_amm_group_destroy(pimdl_amm_group* grp)
+{
+    if (!grp) return PIMDL_OK;
+    (void)hipSetDevice(grp->ctx->device);
+    (void)hipStreamSynchronize(grp->ctx->stream);
+    (void)hipFree(grp->d_centroids);
+    delete grp;
+    return PIMDL_OK;
+}
+
+int pimdl_amm_group_run(pimdl_amm_group* grp, const float* in, uint32_t n, float* const* outs)
+{
+    if (!grp) return PIMDL_ERR_INVALID;
+    Ctx* ctx = grp->ctx;
+    if (!in || !outs) return set_error(ctx, PIMDL_ERR_INVALID, "null buffer");
+    for (size_t i = 0; i < grp->members.size(); ++i)
+        if (!outs[i]) return set_error(ctx, PIMDL_ERR_INVALID, "null output %zu", i);
+    if (n > grp->max_n) return set_error(ctx, PIMDL_ERR_INVALID, "n=%u exceeds max_n=%u of this group", n, grp->max_n);
+    int rc = activate(ctx);
+    if (rc || n == 0) return rc;
+    const float* d_in;
+    if ((rc = stage_input(ctx, grp->members[0]->g, in, n, &d_in))) return rc;
+    if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, idx_buffer_bytes(grp->g, n), "hipMalloc(index scratch)"))) return rc;
+    if ((rc = launch_ccs(ctx, grp->g, d_in, grp->d_centroids, ctx->d_idx, n, grp->x_cols))) return rc;
+    for (size_t i = 0; i < grp->members.size(); ++i) {
+        // member i's index bytes are bytes i*rb .. (i+1)*rb-1 of every row of the common buffer
+        Amm view = *grp->members[i];
+        const size_t rb = view.g.idx_row_bytes;
+        view.g.idx_row_bytes = grp->g.idx_row_bytes;
+        const uint8_t* idx_i = ctx->d_idx + (grp->g.idx_tiled ? i * rb * 64 : i * rb);
+        float* d_out;
+        bool out_host;
+        if ((rc = stage_output(ctx, view.g, outs[i], n, &d_out, &out_host))) return rc;
+        if ((rc = launch_gather(ctx, view, idx_i, d_out, nullptr, n))) return rc;
+        if ((rc = finish_output(ctx, view.g, outs[i], n, out_host))) return rc;
+    }
     return PIMDL_OK;
 }
 

@@ -100,8 +100,11 @@ int set_error(Ctx* ctx, int code, const char* fmt, ...);
 int hip_check(Ctx* ctx, hipError_t e, const char* what);
 
 // kernels (launchers validate nothing: callers have already checked shapes against AmmGeom)
+// x_cols != 0: the geometry's codebooks are those of several operators that all read rows of x_cols
+// floats (g.K = operators * x_cols); only where ccs_supports_shared_input() says so.
 int launch_ccs(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_cent, uint8_t* d_idx,
-               uint32_t n);
+               uint32_t n, uint32_t x_cols = 0);
+bool ccs_supports_shared_input(const AmmGeom& g, uint32_t x_cols);
 // A centroid buffer holds the raw [CB][C][v] floats followed by data derived from them for the
 // search kernel; allocate ccs_centroid_bytes() and run launch_ccs_prep() after every upload.
 size_t ccs_centroid_bytes(const AmmGeom& g);

@@ -265,6 +265,54 @@ def test_two_tokens_per_lane_in_the_fp32_table_gather(ctx, kind):
     amm.close()
 
 
+@pytest.mark.parametrize("N,K,v,C,Ms,lut", [
+    (300, 256, 4, 16, (96, 200, 64), "i8"),     # tiled index rows (matrix-core gather), three outputs of different widths
+    (1000, 128, 4, 8, (128, 128), "i8"),        # paired gather
+    (257, 256, 2, 32, (100, 60), "i8"),         # 32 centroids: byte indices, row-major index rows
+    (300, 256, 8, 16, (48, 80, 48), "f32"),     # fp32 tables
+])
+def test_operators_sharing_an_input_are_searched_by_one_launch(ctx, N, K, v, C, Ms, lut):
+    """AmmGroup (separate Q/K/V projections): every output bit for bit that of the operator run alone."""
+    rng = np.random.default_rng(N + K)
+    x = rng.standard_normal((N, K)).astype(np.float32)
+    amms = []
+    for i, M in enumerate(Ms):
+        _, cent, table, bias = make_case(900 + i, 1, K, v, C, M, lut)
+        amms.append(ctx.amm(cent, table, None if lut == "f32" else np.float32(0.01 * (i + 1)), bias, max_n=N))
+    group = ctx.amm_group(amms)
+    outs = group.run(x)
+    for a, o in zip(amms, outs):
+        assert np.array_equal(o.view(np.uint32), a.run(x).view(np.uint32))
+    outs2 = group.run(x[:77])  # a smaller batch through the same group
+    for o, o2 in zip(outs, outs2):
+        assert np.array_equal(o[:77], o2)
+    group.close()
+    for a in amms:
+        a.close()
+
+
+def test_group_conditions(ctx):
+    rng = np.random.default_rng(5)
+    mk = lambda K, v, C, M, kind="i8": ctx.amm(*(lambda c: (c[1], c[2]))(make_case(1, 1, K, v, C, M, kind)),
+                                               None if kind == "f32" else np.float32(0.01), None, max_n=64)
+    a, b = mk(128, 4, 16, 32), mk(128, 4, 16, 48)
+    for bad in (mk(256, 4, 16, 32), mk(128, 2, 16, 32), mk(128, 4, 8, 32), mk(128, 4, 16, 32, "f32")):
+        with pytest.raises(pimdl.PimdlError):
+            ctx.amm_group([a, bad])
+        bad.close()
+    with pytest.raises(pimdl.PimdlError):
+        ctx.amm_group([a])                       # fewer than two operators
+    c40a, c40b = mk(160, 4, 16, 32), mk(160, 4, 16, 32)  # 40 codebooks: not a multiple of 32
+    with pytest.raises(pimdl.PimdlError):
+        ctx.amm_group([c40a, c40b])
+    g = ctx.amm_group([a, b])
+    with pytest.raises(pimdl.PimdlError):
+        g.run(rng.standard_normal((65, 128)).astype(np.float32))  # beyond max_n
+    g.close()
+    for m in (a, b, c40a, c40b):
+        m.close()
+
+
 def test_scale_groups_from_lutgen(ctx):
     """lutgen with per-group quantisation -> operator with the same grouping: closer to the fp32 product
     than the per-tensor quantisation of the same table, and equal to the oracle on the generated table."""

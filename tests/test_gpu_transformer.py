@@ -62,6 +62,33 @@ def gelu_tanh64(f):
     return 0.5 * f * (1 + np.tanh(math.sqrt(2 / math.pi) * (f + 0.044715 * f ** 3)))
 
 
+def test_qkv_modes_give_the_same_bits(ctx):
+    """Q/K/V as a group (one search launch), on three streams, and one by one."""
+    import torch
+    p = T.TransformerParams(16, 3, 4, 32, 128, 256, 2)  # 32 codebooks per projection: a shared search exists
+    for op, (cb, k_in, m_out) in {"q": (32, 128, 128), "k": (32, 128, 128), "v": (32, 128, 128), "o": (32, 128, 128),
+                                  "ffn1": (32, 128, 256), "ffn2": (64, 256, 128)}.items():
+        p.shapes[op] = T.AmmShape(cb, 16, k_in, m_out)
+    layers = T.synth_layers(p, ctx, pimdl, seed=6)
+    x = torch.randn((p.n, p.token_dim), device="cuda", generator=torch.Generator(device="cuda").manual_seed(2))
+    outs = []
+    for parallel in (False, True):
+        m = T.Transformer(ctx, pimdl, layers, p, parallel_qkv=parallel)
+        assert (m.layers[0].qkv_group is None) == parallel
+        outs.append(m.forward(x).clone())
+        torch.cuda.synchronize()
+        m.close()
+    one = T.TransformerLayer(ctx, pimdl, layers[0], p)
+    one.qkv_group.close()
+    one.qkv_group = None  # falls back to three runs
+    grouped = T.TransformerLayer(ctx, pimdl, layers[0], p)
+    assert torch.equal(one.forward(x), grouped.forward(x))
+    torch.cuda.synchronize()
+    one.close()
+    grouped.close()
+    assert torch.equal(outs[0], outs[1])
+
+
 @pytest.mark.parametrize("fused_gelu", [True, False])
 def test_layer_stage_by_stage(ctx, fused_gelu):
     import torch
