@@ -352,9 +352,9 @@ __global__ __launch_bounds__(CCS_THREADS) void ccs_kernel(const float* __restric
 // each below 2(XX+CN): together with the reference chain's 2(v+2)u(XX+CN) that is below
 // (5v+8)u(XX+CN); the kernel uses twice that.
 // =============================================================================================
-template <int V, bool WIDE = false>
+template <int V, bool WIDE = false, int TTOK = 128>
 struct CcsMfmaShape {
-    static constexpr int TILE_TOKENS = 128;
+    static constexpr int TILE_TOKENS = TTOK;               // 128, or 64 for batches with few tiles
     static constexpr int CBW = 16;                         // codebooks per tile: 2 pairs per wave
     static constexpr int RCB = WIDE ? CBW / 2 : CBW;       // wide: a "pair" is the two 16-centroid halves of one codebook
     static constexpr int TF = RCB * V;                     // floats per tile row
@@ -701,7 +701,7 @@ __global__ void ccs_prep_bf16_kernel(const float* __restrict__ cent, uint4* __re
     }
 }
 
-template <int V, bool WIDE>
+template <int V, bool WIDE, int TTOK>
 __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* __restrict__ x,
                                                                  const float* __restrict__ cent,
                                                                  const uint4* __restrict__ aux_b,
@@ -714,7 +714,7 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
 {
     // K is the length of an activation row.  tiles_x < tiles_cb: the codebooks are those of several operators
     // that read the same row (tiles_x codebook tiles each), so the activation columns wrap around.
-    using S = CcsMfmaShape<V, WIDE>;
+    using S = CcsMfmaShape<V, WIDE, TTOK>;
     constexpr int TF = S::TF, PITCH = S::PITCH, TT = S::TILE_TOKENS, CBW = S::CBW, TG = S::TG, RCB = S::RCB;
     constexpr int XSTEP = WIDE ? V : 2 * V;  // activation floats per pair
     constexpr int NM = (int)ccs_bf16_nm(V);  // MFMAs per item: 2 codebooks x v dims x 6 cross products, 16 K-slots each
@@ -1160,17 +1160,17 @@ static bool ccs_f32_only()
     return v;
 }
 
-template <int V, bool WIDE>
-int launch_ccs_bf16(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_cent, uint8_t* d_idx, uint32_t n,
-                    uint32_t x_cols)
+template <int V, bool WIDE, int TTOK>
+int launch_ccs_bf16_tt(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_cent, uint8_t* d_idx, uint32_t n,
+                       uint32_t x_cols)
 {
-    using S = CcsMfmaShape<V, WIDE>;
+    using S = CcsMfmaShape<V, WIDE, TTOK>;
     const uint32_t tiles_cb = g.CB_pad / S::RCB;  // CB_pad is a multiple of 32
     const uint64_t total64 = (uint64_t)((n + S::TILE_TOKENS - 1) / S::TILE_TOKENS) * tiles_cb;
     if (total64 > 0xFFFFFFFFull) return set_error(ctx, PIMDL_ERR_INVALID, "ccs: too many tiles");
     const uint32_t total = (uint32_t)total64;
     int per_cu = 0;  // persistent grid: exactly the workgroups that are resident at once
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, ccs_bf16_kernel<V, WIDE>, CCS_THREADS, 0) != hipSuccess || per_cu < 1) {
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, ccs_bf16_kernel<V, WIDE, TTOK>, CCS_THREADS, 0) != hipSuccess || per_cu < 1) {
         (void)hipGetLastError();
         per_cu = 1;
     }
@@ -1185,9 +1185,22 @@ int launch_ccs_bf16(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d
     const float* bf = d_cent + ccs_bf16_offset(g);
     const uint4* aux_b = reinterpret_cast<const uint4*>(bf);
     const float* cn16 = bf + ccs_bf16_units(g) * ccs_bf16_nm(V) * 64 * 4;
-    hipLaunchKernelGGL((ccs_bf16_kernel<V, WIDE>), grid, dim3(CCS_THREADS), 0, ctx->stream, d_x, d_cent, aux_b, cn16, cnmax_pad,
+    hipLaunchKernelGGL((ccs_bf16_kernel<V, WIDE, TTOK>), grid, dim3(CCS_THREADS), 0, ctx->stream, d_x, d_cent, aux_b, cn16, cnmax_pad,
                        d_idx, n, row, g.CB, g.C, g.idx_row_bytes, (int)g.idx_tiled, vec_ok, tiles_cb, total, tiles_x);
     return hip_check(ctx, hipGetLastError(), "ccs_bf16_kernel launch");
+}
+
+// 128-token tiles amortise a tile's operand loads best, but a workgroup that gets only one or two of them
+// cannot overlap a tile's loads with the previous tile's arithmetic: small batches use 64-token tiles.
+template <int V, bool WIDE>
+int launch_ccs_bf16(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_cent, uint8_t* d_idx, uint32_t n,
+                    uint32_t x_cols)
+{
+    const uint64_t tiles128 = (uint64_t)((n + 127) / 128) * (g.CB_pad / CcsMfmaShape<V, WIDE>::RCB);
+    // (measured: 7.4 -> 5.9 us at 192 tiles, 8.7 -> 6.9 us at 384, equal at 768 = one per resident workgroup,
+    // 10 % slower beyond)
+    if (tiles128 < 3ull * ctx->prop.multiProcessorCount) return launch_ccs_bf16_tt<V, WIDE, 64>(ctx, g, d_x, d_cent, d_idx, n, x_cols);
+    return launch_ccs_bf16_tt<V, WIDE, 128>(ctx, g, d_x, d_cent, d_idx, n, x_cols);
 }
 
 template <int IDX_BITS>
