@@ -26,8 +26,8 @@ HBM_PEAK_GBPS = 8000.0                     # MI355X HBM3E
 # WRITE_SIZE by 1.0: the factors a streaming kernel of known size gives for the same counters on
 # this part.  Summary: profiles/bench_ffn_pair_hbm_traffic.txt.  Keyed by (K, M).
 MEASURED_GATHER_TRAFFIC = {
-    (768, 3072): {"fetch_kib": 7997.7, "write_kib": 111227.3},
-    (3072, 768): {"fetch_kib": 15534.9, "write_kib": 26639.7},
+    (768, 3072): {"fetch_kib": 7992.3, "write_kib": 111172.0},
+    (3072, 768): {"fetch_kib": 15578.0, "write_kib": 26636.7},
 }
 FETCH_SCALE, WRITE_SCALE = 2.0, 1.0
 LDS_PEAK_GBPS = 256 * 256 * 2.4            # 256 CUs x 256 B/clk (ds_read_b128) x 2.4 GHz = 157286 GB/s
