@@ -6,10 +6,14 @@
 //     acc[n][f] = sum over cb of lut[cb][idx[n][cb]][f]          (int8 table, int32 sum, exact)
 //     out[n][f] = (float)acc * scale + lut_bias(*CB) + bias[f]   (fp32, left to right, unfused)
 //
-// The path is bound by LDS read bandwidth: every gathered LUT byte is read once from LDS
-// (N*CB*M bytes), while HBM only sees the packed indices, the LUT slices and the output.
+// Three kernels: the one-hot matrix-core gather for int8 tables with up to 16 centroids (further down,
+// the one the benchmark shapes run), the byte adder below for int8 tables with more centroids, and the
+// fp32-table gather (also used for int8 tables with one scale per group of codebooks).
 //
-// int8 kernel.  A workgroup owns a tile of tokens x one column block (16*Q columns) and walks the
+// The byte adder and the fp32 gather are bound by LDS read bandwidth: every gathered LUT byte is read
+// once from LDS (N*CB*M bytes), while HBM only sees the packed indices, the LUT slices and the output.
+//
+// int8 byte adder.  A workgroup owns a tile of tokens x one column block (16*Q columns) and walks the
 // codebooks in slices that are staged into LDS (double buffered; the next slice is fetched into
 // registers while the current one is consumed).  Inside a wave, lane l = 16*g + j works for token j
 // of a 16-token group and for the g-th quarter of the slice's codebooks: it turns its 4/8-bit index
