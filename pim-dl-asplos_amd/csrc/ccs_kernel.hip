@@ -1169,10 +1169,16 @@ int launch_ccs_bf16_tt(Ctx* ctx, const AmmGeom& g, const float* d_x, const float
     const uint64_t total64 = (uint64_t)((n + S::TILE_TOKENS - 1) / S::TILE_TOKENS) * tiles_cb;
     if (total64 > 0xFFFFFFFFull) return set_error(ctx, PIMDL_ERR_INVALID, "ccs: too many tiles");
     const uint32_t total = (uint32_t)total64;
-    int per_cu = 0;  // persistent grid: exactly the workgroups that are resident at once
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, ccs_bf16_kernel<V, WIDE, TTOK>, CCS_THREADS, 0) != hipSuccess || per_cu < 1) {
-        (void)hipGetLastError();
-        per_cu = 1;
+    // persistent grid: exactly the workgroups that are resident at once (asked once per kernel variant;
+    // every device this library runs on is the same part)
+    static int per_cu = 0;
+    if (per_cu == 0) {
+        int q = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&q, ccs_bf16_kernel<V, WIDE, TTOK>, CCS_THREADS, 0) != hipSuccess || q < 1) {
+            (void)hipGetLastError();
+            q = 1;
+        }
+        per_cu = q;
     }
     const uint32_t slots = (uint32_t)ctx->prop.multiProcessorCount * (uint32_t)per_cu;
     dim3 grid(total < slots ? total : slots);
