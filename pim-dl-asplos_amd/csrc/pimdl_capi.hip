@@ -119,14 +119,21 @@ static int check_run_args(Amm* amm, const void* a, const void* b, uint32_t n)
 template <typename T>
 static void retile_lut(const T* lut, T* tiled, const AmmGeom& g, uint32_t row_elems)
 {
-    // canonical [CB][C][M] -> [M_pad/row_elems][CB_pad][C_tile][row_elems], zero padded
+    // canonical [CB][C][M] -> [M_pad/row_elems][CB_pad][C_tile][row_elems], zero padded;
+    // chunked fp32 tables: [M_pad/row_elems][CB_pad][row_elems/2][C_tile][2]
     const uint32_t nblk = g.M_pad / row_elems;
+    const bool chunked = sizeof(T) == 4 && g.lut_chunked;
     for (uint32_t b = 0; b < nblk; ++b)
         for (uint32_t cb = 0; cb < g.CB; ++cb)
             for (uint32_t c = 0; c < g.C; ++c) {
                 const T* src = lut + ((size_t)cb * g.C + c) * g.M + (size_t)b * row_elems;
-                T* dst = tiled + (((size_t)b * g.CB_pad + cb) * g.C_tile + c) * row_elems;
                 const uint32_t cnt = (b + 1) * row_elems <= g.M ? row_elems : g.M - b * row_elems;
+                if (chunked) {
+                    T* blk = tiled + ((size_t)b * g.CB_pad + cb) * g.C_tile * row_elems;
+                    for (uint32_t e = 0; e < cnt; ++e) blk[((size_t)(e / 2) * g.C_tile + c) * 2 + e % 2] = src[e];
+                    continue;
+                }
+                T* dst = tiled + (((size_t)b * g.CB_pad + cb) * g.C_tile + c) * row_elems;
                 memcpy(dst, src, sizeof(T) * cnt);
             }
 }

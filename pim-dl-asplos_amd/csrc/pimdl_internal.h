@@ -29,6 +29,7 @@ struct AmmGeom {
     uint32_t K, v, CB, CB_pad, C, C_tile, M, M_pad;
     uint32_t idx_bits, idx_row_bytes;
     uint32_t idx_tiled;     // layout of the packed index buffer, see above
+    uint32_t lut_chunked;   // fp32 table of 32 centroids: [column block][codebook][8-byte chunk][row][2 floats]
     // gather kernel
     uint32_t gather_kind;   // 0: byte-adder rows kernel, 1: one-hot matrix-core kernel (int8, C <= 16)
     uint32_t q;             // 16-byte chunks per LUT row in LDS
@@ -40,6 +41,9 @@ struct AmmGeom {
     // ccs kernel
     uint32_t ccs_row_floats, ccs_cb_per_wg, ccs_lds_bytes;
 };
+
+// fp32 tables whose rows are read in 8-byte chunks (see gather_f32_kernel)
+constexpr bool f32_lut_chunked(int c_tile, int q) { return c_tile == 32 && q == 4; }
 
 // bytes of a packed index buffer for n tokens
 inline size_t idx_buffer_bytes(const AmmGeom& g, uint32_t n)
