@@ -295,7 +295,7 @@ class Transformer:
     def capture(self, x):
         """Records one forward pass on `x`'s shape into a HIP graph and returns (graph, static_input,
         static_output): copy new features into static_input, graph.replay(), read static_output.
-        A layer is ~30 short kernels; launched one by one from Python the GPU waits for the host
+        A layer is ~20 short kernels; launched one by one from Python the GPU waits for the host
         about a third of the time, replayed from a graph it does not.  The library's calls are
         recorded like any other launch (they run on the stream the context is bound to and, for
         device buffers that have been seen before, allocate and synchronise nothing)."""
@@ -348,17 +348,21 @@ def synth_layers(params, ctx, pimdl, seed=0, shared_qkv_centroids=False):
 
 def main(argv=None):
     """Counterpart of the reference's test_transformer driver:
-        python transformer.py config.yaml [weights.npz] [--iters K]
+        python transformer.py config.yaml [weights.npz] [--iters K] [--graph]
     reads the same YAML and weight file, runs the model forward on random token features and prints
-    the per-iteration time in the reference's wording (test_transformer.cpp:356)."""
+    the per-iteration time in the reference's wording (test_transformer.cpp:356).  --graph records the
+    forward once into a HIP graph and times its replays (no host work between the kernels)."""
     argv = list(sys.argv[1:] if argv is None else argv)
     iters = 5
+    use_graph = "--graph" in argv
+    if use_graph:
+        argv.remove("--graph")
     if "--iters" in argv:
         i = argv.index("--iters")
         iters = int(argv[i + 1])
         del argv[i:i + 2]
     if not argv:
-        print("usage: transformer.py config_yaml_path [weight_path] [--iters K]", file=sys.stderr)
+        print("usage: transformer.py config_yaml_path [weight_path] [--iters K] [--graph]", file=sys.stderr)
         return 2
     here = os.path.dirname(os.path.abspath(__file__))
     sys.path.insert(0, os.path.dirname(here))
@@ -378,11 +382,17 @@ def main(argv=None):
     model = Transformer(ctx, pimdl, layers, params)
     print("finish weight initialization")
     x = torch.randn((params.n, params.token_dim), device="cuda", dtype=torch.float32)
+    if use_graph:
+        graph, static_x, _static_y = model.capture(x)
     print("inference start")
     for i in range(iters):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        model.forward(x)
+        if use_graph:
+            static_x.copy_(x)
+            graph.replay()
+        else:
+            model.forward(x)
         torch.cuda.synchronize()
         print(f"iteration {i}, inference time {time.perf_counter() - t0:.6f}")
     print("inference end")

@@ -201,6 +201,8 @@ def test_driver_prints_the_reference_wording(capsys):
     out = capsys.readouterr().out
     assert "weight file is not found, generate weights randomly." in out
     assert "iteration 1, inference time" in out and "inference end" in out
+    assert T.main([CFG, "--iters", "2", "--graph"]) == 0  # the same through a recorded HIP graph
+    assert "iteration 1, inference time" in capsys.readouterr().out
 
 
 def test_column_tile_hint_and_measured_tile_search(ctx, tmp_path):
