@@ -455,3 +455,50 @@ def test_search_at_full_ffn2_shape(ctx):
         got = amm.index_calculation(x)
         assert np.array_equal(got, want), f"{dist}: {(got != want).sum()} of {got.size} differ"
         amm.close()
+
+
+def _random_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for i in range(count):
+        v = int(rng.choice([2, 4, 8, 2, 4, 8, 3, 16]))
+        C = int(rng.choice([rng.integers(2, 9), rng.integers(9, 17), rng.integers(17, 33), 16, 16, 32, 8, 64]))
+        CB = int(rng.choice([rng.integers(1, 12), rng.integers(12, 80), 32, 64, 96]))
+        M = int(rng.choice([rng.integers(1, 64), rng.integers(64, 420), 96, 192, 768]))
+        N = int(rng.choice([rng.integers(1, 70), rng.integers(70, 700), rng.integers(700, 2600), 256, 1024]))
+        kind = str(rng.choice(["i8", "i8", "i8", "f32", "grouped"]))
+        cases.append((i, N, CB * v, v, C, M, kind))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_cases(48, 2024), ids=lambda c: "n%d_k%d_v%d_c%d_m%d_%s" % c[1:])
+def test_random_shapes_against_the_oracle(ctx, case):
+    """Seeded random shapes across every kernel variant (search: bf16 narrow / wide, exact, generic; gather:
+    one-hot, paired, byte adder, fp32 one and two tokens per lane, grouped), with a non-zero LUT bias in both
+    bias modes for the int8 table."""
+    i, N, K, v, C, M, kind = case
+    x, cent, lut, bias = make_case(7000 + i, N, K, v, C, M, "f32" if kind == "f32" else "i8")
+    CB = K // v
+    want_idx = oracle.index_calculation(x, cent, v, threads=THREADS)
+    if kind == "i8":
+        mode = i % 2
+        amm = ctx.amm(cent, lut, np.float32(0.0371), bias, max_n=N, lut_bias=0.25, bias_mode=mode)
+        out, idx, acc = amm.run_debug(x)
+        want_acc = oracle.gather_i8(want_idx, lut, threads=THREADS)
+        assert np.array_equal(idx, want_idx)
+        assert np.array_equal(acc, want_acc)
+        want = oracle.dequant(want_acc, bias, CB, 0.0371, 0.25, mode, threads=THREADS)
+        assert np.array_equal(out.view(np.uint32), want.view(np.uint32))
+    elif kind == "f32":
+        amm = ctx.amm(cent, lut, None, bias, max_n=N)
+        out, idx, _ = amm.run_debug(x)
+        assert np.array_equal(idx, want_idx)
+        np.testing.assert_allclose(out, oracle.gather_f32(want_idx, lut, bias, threads=THREADS), rtol=1e-5,
+                                   atol=1e-5 * np.sqrt(CB))
+    else:
+        group = 1 + i % 5
+        scales = np.random.default_rng(i).uniform(1e-3, 0.1, (CB + group - 1) // group).astype(np.float32)
+        amm = ctx.amm(cent, lut, scales, bias, max_n=N, scale_group=group)
+        want = oracle.gather_i8_grouped(want_idx, lut, scales, bias, group, threads=THREADS)
+        assert np.array_equal(amm.run(x).view(np.uint32), want.view(np.uint32))
+    amm.close()
