@@ -86,7 +86,7 @@ def model_forward(pimdl, ctx, iters=10):
     model.close()
     return {"layers": 12, "tokens": p.n, "ms_per_forward": ms, "tokens_per_s": p.n / (ms * 1e-3),
             "ms_per_forward_graph": ms_graph, "tokens_per_s_graph": p.n / (ms_graph * 1e-3),
-            "note": "LUT-AMM linears (tanh-GELU inside the first feed-forward operator's epilogue) + pimdl_layer_norm on libpimdl, attention in PyTorch-ROCm fp32"}
+            "note": "LUT-AMM linears (tanh-GELU inside the first feed-forward operator's epilogue), pimdl_layer_norm and pimdl_attention (fp32) on libpimdl; PyTorch-ROCm for tensors, streams and graph capture"}
 
 
 def cpu_baseline(shapes, N, budget_s=12.0):

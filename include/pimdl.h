@@ -226,6 +226,18 @@ PIMDL_API int pimdl_lutgen(pimdl_ctx* ctx, const float* centroids, const float* 
 PIMDL_API int pimdl_layer_norm(pimdl_ctx* ctx, const float* x, const float* weight, const float* bias,
                                const float* residual, float* out, uint32_t n, uint32_t d, float eps);
 
+/* ---- attention of the transformer layer ---------------------------------------------------------
+ * Replaces step 2 of the reference's attention (src/host/transformer_layer.cpp:211-230: K Q, scale,
+ * soft_max, V KQ, permute back), unmasked, fp32:  out = softmax(q k^T * scale) v  per (batch, head).
+ *   q, k, v  DEVICE fp32 [batch*seq][in_stride], head h in columns 64 h .. 64 h + 63 (three column
+ *            ranges of one fused [n][3*token_dim] buffer are fine: pass the three start addresses)
+ *   out      DEVICE fp32 [batch*seq][out_stride], same column order: no head transposes
+ * head_dim must be 64 (PIMDL_ERR_UNSUPPORTED otherwise: the caller keeps its own attention then).
+ * Queued on the context's stream. */
+PIMDL_API int pimdl_attention(pimdl_ctx* ctx, const float* q, const float* k, const float* v, float* out,
+                              uint32_t batch, uint32_t seq, uint32_t heads, uint32_t head_dim,
+                              uint32_t in_stride, uint32_t out_stride, float scale);
+
 /* ---- introspection ---------------------------------------------------------------------------
  * No reference counterpart: figures a benchmark needs to place a kernel on its roofline. */
 typedef struct pimdl_device_info {

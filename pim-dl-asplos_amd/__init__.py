@@ -30,7 +30,8 @@ EXPORTS = ["pimdl_init", "pimdl_destroy", "pimdl_last_error", "pimdl_set_stream"
            "pimdl_amm_profile", "pimdl_index_calculation", "pimdl_amm_index_calculation", "pimdl_lut_gather",
            "pimdl_amm_run_tiled", "pimdl_lut_gather_tiled", "pimdl_lutgen",
            "pimdl_layer_norm", "pimdl_get_device_info", "pimdl_amm_get_geometry", "pimdl_diag_bandwidth",
-           "pimdl_diag_mfma_error", "pimdl_amm_group_create", "pimdl_amm_group_run", "pimdl_amm_group_destroy"]
+           "pimdl_diag_mfma_error", "pimdl_amm_group_create", "pimdl_amm_group_run", "pimdl_amm_group_destroy",
+           "pimdl_attention"]
 
 
 class PimdlError(RuntimeError):
@@ -131,6 +132,7 @@ def lib():
     L.pimdl_amm_group_create.argtypes = [vp, ctypes.POINTER(vp), u32, ctypes.POINTER(vp)]
     L.pimdl_amm_group_run.argtypes = [vp, vp, u32, ctypes.POINTER(vp)]
     L.pimdl_amm_group_destroy.argtypes = [vp]
+    L.pimdl_attention.argtypes = [vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, ctypes.c_float]
     for name in EXPORTS:
         if name != "pimdl_last_error":
             getattr(L, name).restype = ctypes.c_int
@@ -242,6 +244,12 @@ class Context:
         self._check(lib().pimdl_layer_norm(self._h, _ptr(x), _ptr(weight), _ptr(bias), _ptr(residual), _ptr(y), n, d,
                                            ctypes.c_float(eps)))
         return y
+
+    def attention_ptr(self, q, k, v, out, batch, seq, heads, head_dim, in_stride, out_stride, scale):
+        """Device addresses; out = softmax(q k^T * scale) v per (batch, head), unmasked (head_dim 64 only)."""
+        self._check(lib().pimdl_attention(self._h, ctypes.c_void_p(q), ctypes.c_void_p(k), ctypes.c_void_p(v),
+                                          ctypes.c_void_p(out), batch, seq, heads, head_dim, in_stride, out_stride,
+                                          ctypes.c_float(scale)))
 
     def amm_group(self, amms):
         return AmmGroup(self, amms)

@@ -858,7 +858,9 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
             });
 #pragma unroll
             for (int t = 0; t < TM; ++t) {
-                const uint32_t entry = P8 ? iwm[t][ks] : __builtin_amdgcn_ubfe(iwm[t][ks / 2], 16 * (ks & 1) + byte_shift, 8);
+                uint32_t entry;
+                if constexpr (P8) entry = iwm[t][ks];
+                else entry = __builtin_amdgcn_ubfe(iwm[t][ks / 2], 16 * (ks & 1) + byte_shift, 8);
                 lds_read<0>(b_op[ks & 1][t], entry);
             }
         };
@@ -1057,7 +1059,7 @@ __global__ __launch_bounds__(GF_THREADS) void gather_f32_kernel(const uint8_t* _
 #pragma unroll
             for (int t = 0; t < TPL; ++t) word[t] = idx_cur[t][w];
             // ascending codebook order; partial unroll keeps the loads in flight within the VGPR budget
-#pragma unroll(TPL == 1 ? 4 : 2)
+#pragma unroll 2
             for (int h = 0; h < per_word; ++h) {
 #pragma unroll
                 for (int t = 0; t < TPL; ++t) {

@@ -720,6 +720,25 @@ int pimdl_amm_get_geometry(const pimdl_amm* a, pimdl_amm_geometry* out)
     return PIMDL_OK;
 }
 
+int pimdl_attention(pimdl_ctx* ctx, const float* q, const float* k, const float* v, float* out, uint32_t batch,
+                    uint32_t seq, uint32_t heads, uint32_t head_dim, uint32_t in_stride, uint32_t out_stride, float scale)
+{
+    if (!ctx) return PIMDL_ERR_INVALID;
+    if (!q || !k || !v || !out) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_attention: null buffer");
+    if (head_dim != 64) return set_error(ctx, PIMDL_ERR_UNSUPPORTED, "pimdl_attention: head_dim=%u (only 64 is built)", head_dim);
+    if (batch > 65535 || heads > 65535) return set_error(ctx, PIMDL_ERR_UNSUPPORTED, "pimdl_attention: batch and heads must be below 65536");
+    if ((uint64_t)heads * 64 > in_stride || (uint64_t)heads * 64 > out_stride || in_stride % 4 || out_stride % 4)
+        return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_attention: strides must hold heads*64 floats and be multiples of 4");
+    if (!is_device_ptr(q) || !is_device_ptr(k) || !is_device_ptr(v) || !is_device_ptr(out))
+        return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_attention: q, k, v and out must be device pointers");
+    if ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) | reinterpret_cast<uintptr_t>(v) |
+         reinterpret_cast<uintptr_t>(out)) & 15)
+        return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_attention: pointers must be 16-byte aligned");
+    int rc = activate(ctx);
+    if (rc) return rc;
+    return launch_attention_hd64(ctx, q, k, v, out, batch, seq, heads, in_stride, out_stride, scale);
+}
+
 int pimdl_layer_norm(pimdl_ctx* ctx, const float* x, const float* weight, const float* bias, const float* residual,
                      float* out, uint32_t n, uint32_t d, float eps)
 {

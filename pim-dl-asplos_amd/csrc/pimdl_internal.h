@@ -128,6 +128,8 @@ int launch_lut_quant(Ctx* ctx, const float* d_lut, int8_t* d_q, float* d_scales,
                      uint32_t M, uint32_t scale_group);
 int launch_layer_norm(Ctx* ctx, const float* d_x, const float* d_w, const float* d_b, const float* d_residual,
                       float* d_out, uint32_t n, uint32_t d, float eps);
+int launch_attention_hd64(Ctx* ctx, const float* d_q, const float* d_k, const float* d_v, float* d_out, uint32_t batch,
+                          uint32_t seq, uint32_t heads, uint32_t in_stride, uint32_t out_stride, float scale);
 int launch_diag(Ctx* ctx, uint64_t bytes, float* copy_gbps, float* lds_gbps);
 int launch_diag_mfma_error(Ctx* ctx, uint32_t trials, float* max_err_u);
 

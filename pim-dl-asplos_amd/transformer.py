@@ -10,10 +10,10 @@ Host-side counterpart of the reference's layer/model code (C++ over ggml and the
 
 Every linear layer is a LUT-AMM operator of libpimdl (closest-centroid search + LUT gather on the GPU);
 layer normalisation is libpimdl's pimdl_layer_norm (the reference's norm() statement by statement);
-attention and the activation are PyTorch-ROCm fp32 operations on the same stream.  The reference computes
-those two with ggml (flash attention, GELU through an fp16 table); no test of the reference pins their
-outputs, so here they are the textbook definitions: softmax(Q K^T / sqrt(head_dim)) V without a mask, and
-the tanh form of GELU.  The DPU tile re-orderings between the steps of the reference layer disappear:
+attention is libpimdl's pimdl_attention for head_dim 64 (PyTorch-ROCm's fused attention otherwise) and GELU
+runs inside the first feed-forward operator's epilogue.  The reference computes those two with ggml (flash
+attention, GELU through an fp16 table); no test of the reference pins their outputs, so here they are the
+textbook fp32 definitions: softmax(Q K^T / sqrt(head_dim)) V without a mask, and the tanh form of GELU.  The DPU tile re-orderings between the steps of the reference layer disappear:
 every buffer here is row-major [tokens][features].
 
 Op order of one layer (transformer_layer.cpp, "step" comments):
@@ -160,6 +160,7 @@ class TransformerLayer:
         self.ctx, self.params, self.torch = ctx, params, torch
         self.fused_qkv = fused_qkv
         self.fused_gelu = fused_gelu
+        self.own_attention = True  # head_dim 64: pimdl_attention; other head sizes use PyTorch's fused attention
         self.side = None if fused_qkv else side
         n = params.n
         self.amm = {}
@@ -243,12 +244,18 @@ class TransformerLayer:
                 main.wait_stream(stream)                                   # join
         else:
             q, k, v = self._run("q", x, n), self._run("k", x, n), self._run("v", x, n)
-        qh, kh, vh = (t.reshape(B, S, H, hd).permute(0, 2, 1, 3) for t in (q, k, v))
-        # unmasked softmax(q k^T / sqrt(head_dim)) v in fp32; the fused kernel reads the strided head views
-        # directly (separate matmul / softmax calls first copy each of them into [B][H][S][hd] order)
-        attn = torch.nn.functional.scaled_dot_product_attention(
-            qh, kh, vh, scale=1.0 / math.sqrt(p.token_dim / p.head_num))     # [B][H][S][hd]
-        a = attn.permute(0, 2, 1, 3).reshape(n, p.token_dim).contiguous()
+        att_scale = 1.0 / math.sqrt(p.token_dim / p.head_num)
+        if hd == 64 and self.own_attention:
+            # the library's attention kernel reads q, k, v where they are (also as column ranges of the fused
+            # projection's output) and writes [n][token_dim] directly
+            a = torch.empty((n, p.token_dim), device=x.device, dtype=torch.float32)
+            self.ctx.attention_ptr(q.data_ptr(), k.data_ptr(), v.data_ptr(), a.data_ptr(), B, S, H, hd,
+                                   q.stride(0), p.token_dim, att_scale)
+        else:
+            qh, kh, vh = (t.reshape(B, S, H, hd).permute(0, 2, 1, 3) for t in (q, k, v))
+            # unmasked softmax(q k^T / sqrt(head_dim)) v in fp32; PyTorch's fused kernel reads the strided head views
+            attn = torch.nn.functional.scaled_dot_product_attention(qh, kh, vh, scale=att_scale)     # [B][H][S][hd]
+            a = attn.permute(0, 2, 1, 3).reshape(n, p.token_dim).contiguous()
         o = self._run("o", a, n)
         h = self._norm_residual("attention_norm", o, x)
         if self.fused_gelu:

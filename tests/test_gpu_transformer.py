@@ -62,10 +62,41 @@ def gelu_tanh64(f):
     return 0.5 * f * (1 + np.tanh(math.sqrt(2 / math.pi) * (f + 0.044715 * f ** 3)))
 
 
+@pytest.mark.parametrize("B,S,H,fused", [(2, 16, 3, False), (3, 128, 4, False), (2, 197, 2, True), (1, 300, 1, False),
+                                          (2, 64, 2, True), (1, 1, 1, False)])
+def test_attention_kernel_against_float64(ctx, B, S, H, fused):
+    """pimdl_attention (head_dim 64, fp32 matrix cores, streaming softmax over 128-key chunks) against
+    softmax(q k^T / 8) v in float64, and against PyTorch's fused attention; also reading q, k, v as three
+    column ranges of one [n][3*token_dim] buffer."""
+    import torch
+    D, n = H * 64, B * S
+    gen = torch.Generator(device="cuda").manual_seed(B * 1000 + S)
+    if fused:
+        qkv = torch.randn((n, 3 * D), device="cuda", generator=gen) * 2.0
+        q, k, v = qkv[:, :D], qkv[:, D:2 * D], qkv[:, 2 * D:]
+        in_stride = 3 * D
+    else:
+        q, k, v = (torch.randn((n, D), device="cuda", generator=gen) * 2.0 for _ in range(3))
+        in_stride = D
+    out = torch.full((n, D), float("nan"), device="cuda")
+    ctx.attention_ptr(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), B, S, H, 64, in_stride, D, 0.125)
+    torch.cuda.synchronize()
+    q64, k64, v64 = (t.double().reshape(B, S, H, 64).permute(0, 2, 1, 3) for t in (q, k, v))
+    p = torch.softmax(q64 @ k64.transpose(-1, -2) * 0.125, dim=-1)
+    want = (p @ v64).permute(0, 2, 1, 3).reshape(n, D)
+    assert not torch.isnan(out).any()
+    torch.testing.assert_close(out.double(), want, rtol=1e-5, atol=1e-5)
+    sd = torch.nn.functional.scaled_dot_product_attention(
+        *(t.reshape(B, S, H, 64).permute(0, 2, 1, 3) for t in (q, k, v)), scale=0.125).permute(0, 2, 1, 3).reshape(n, D)
+    torch.testing.assert_close(out, sd, rtol=1e-4, atol=1e-4)
+    with pytest.raises(pimdl.PimdlError):  # other head sizes are not built
+        ctx.attention_ptr(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), B, S, H, 32, in_stride, D, 0.125)
+
+
 def test_qkv_modes_give_the_same_bits(ctx):
     """Q/K/V as a group (one search launch), on three streams, and one by one."""
     import torch
-    p = T.TransformerParams(16, 3, 4, 32, 128, 256, 2)  # 32 codebooks per projection: a shared search exists
+    p = T.TransformerParams(16, 3, 2, 64, 128, 256, 2)  # 32 codebooks per projection: a shared search exists
     for op, (cb, k_in, m_out) in {"q": (32, 128, 128), "k": (32, 128, 128), "v": (32, 128, 128), "o": (32, 128, 128),
                                   "ffn1": (32, 128, 256), "ffn2": (64, 256, 128)}.items():
         p.shapes[op] = T.AmmShape(cb, 16, k_in, m_out)
@@ -83,6 +114,13 @@ def test_qkv_modes_give_the_same_bits(ctx):
     one.qkv_group = None  # falls back to three runs
     grouped = T.TransformerLayer(ctx, pimdl, layers[0], p)
     assert torch.equal(one.forward(x), grouped.forward(x))
+    # head_dim 64: the library's attention kernel inside the layer against PyTorch's on the same q, k, v
+    keep_own, keep_torch = {}, {}
+    grouped.forward(x, keep_own)
+    grouped.own_attention = False
+    grouped.forward(x, keep_torch)
+    assert torch.equal(keep_own["q"], keep_torch["q"])
+    torch.testing.assert_close(keep_own["attn"], keep_torch["attn"], rtol=1e-4, atol=1e-4)
     torch.cuda.synchronize()
     one.close()
     grouped.close()
