@@ -160,6 +160,15 @@ PIMDL_API int pimdl_amm_group_create(pimdl_ctx* ctx, pimdl_amm* const* amms, uin
                                      pimdl_amm_group** out);
 PIMDL_API int pimdl_amm_group_run(pimdl_amm_group* group, const float* in, uint32_t n, float* const* outs);
 PIMDL_API int pimdl_amm_group_destroy(pimdl_amm_group* group);
+/* When the members are int8 operators of one shape served by the matrix-core gather (up to 16
+ * centroids, output_feature_len a multiple of the column tile, same LUT bias and activation), the
+ * group can also run ONE gather launch over all of them and write one buffer
+ *   out fp32 [n][count * M], operator i in columns i*M .. (i+1)*M - 1
+ * (the layout of the reference's fused qkv output, src/host/transformer_layer.cpp:301), each column
+ * bit for bit that of the operator run alone.  pimdl_amm_group_fused_cols gives count * M, or 0 when
+ * the members do not allow it (pimdl_amm_group_run_fused then returns PIMDL_ERR_UNSUPPORTED). */
+PIMDL_API int pimdl_amm_group_fused_cols(const pimdl_amm_group* group, uint32_t* cols);
+PIMDL_API int pimdl_amm_group_run_fused(pimdl_amm_group* group, const float* in, uint32_t n, float* out);
 
 /* Runs the two kernels `iters` times each on device-resident buffers and reports the average
  * device time of each.  in/out must be DEVICE pointers. */

@@ -31,7 +31,7 @@ EXPORTS = ["pimdl_init", "pimdl_destroy", "pimdl_last_error", "pimdl_set_stream"
            "pimdl_amm_run_tiled", "pimdl_lut_gather_tiled", "pimdl_lutgen",
            "pimdl_layer_norm", "pimdl_get_device_info", "pimdl_amm_get_geometry", "pimdl_diag_bandwidth",
            "pimdl_diag_mfma_error", "pimdl_amm_group_create", "pimdl_amm_group_run", "pimdl_amm_group_destroy",
-           "pimdl_attention"]
+           "pimdl_attention", "pimdl_amm_group_fused_cols", "pimdl_amm_group_run_fused"]
 
 
 class PimdlError(RuntimeError):
@@ -132,6 +132,8 @@ def lib():
     L.pimdl_amm_group_create.argtypes = [vp, ctypes.POINTER(vp), u32, ctypes.POINTER(vp)]
     L.pimdl_amm_group_run.argtypes = [vp, vp, u32, ctypes.POINTER(vp)]
     L.pimdl_amm_group_destroy.argtypes = [vp]
+    L.pimdl_amm_group_fused_cols.argtypes = [vp, ctypes.POINTER(u32)]
+    L.pimdl_amm_group_run_fused.argtypes = [vp, vp, u32, vp]
     L.pimdl_attention.argtypes = [vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, ctypes.c_float]
     for name in EXPORTS:
         if name != "pimdl_last_error":
@@ -271,6 +273,9 @@ class AmmGroup:
         handles = (ctypes.c_void_p * len(self.amms))(*[a._h for a in self.amms])
         self._h = ctypes.c_void_p()
         ctx._check(lib().pimdl_amm_group_create(ctx._h, handles, len(self.amms), ctypes.byref(self._h)))
+        cols = ctypes.c_uint32(0)
+        ctx._check(lib().pimdl_amm_group_fused_cols(self._h, ctypes.byref(cols)))
+        self.fused_cols = int(cols.value)  # > 0: run_fused writes one [n][fused_cols] buffer with one gather launch
 
     def close(self):
         if self._h and self.ctx._h:
@@ -289,6 +294,15 @@ class AmmGroup:
         """Raw addresses (device or host); asynchronous for device memory."""
         ptrs = (ctypes.c_void_p * len(out_ptrs))(*out_ptrs)
         self.ctx._check(lib().pimdl_amm_group_run(self._h, ctypes.c_void_p(in_ptr), n, ptrs))
+
+    def run_fused(self, x):
+        x = np.ascontiguousarray(x, np.float32)
+        out = np.empty((x.shape[0], self.fused_cols), np.float32)
+        self.ctx._check(lib().pimdl_amm_group_run_fused(self._h, _ptr(x), x.shape[0], _ptr(out)))
+        return out
+
+    def run_fused_ptr(self, in_ptr, n, out_ptr):
+        self.ctx._check(lib().pimdl_amm_group_run_fused(self._h, ctypes.c_void_p(in_ptr), n, ctypes.c_void_p(out_ptr)))
 
 
 class Amm:

@@ -57,6 +57,11 @@ struct Epilogue {
     float lut_bias_term;  // lut_bias or lut_bias*CB, already rounded to fp32 like the reference does
     const float* bias;    // [M] or nullptr
     uint32_t act;         // pimdl_activation
+    // Several operators side by side in one launch (one-hot kernel only): column tiles
+    // k * op_col_tiles .. (k+1) * op_col_tiles - 1 belong to operator k, which has its own scale and whose
+    // index bytes start op_idx_stride * k bytes into the index buffer.  op_col_tiles == 0: one operator.
+    const float* op_scales;
+    uint32_t op_col_tiles, op_idx_stride;
 };
 
 // How the items (column tile x token tile) of a gather are dealt to the 8 XCDs.  Workgroup b takes
@@ -639,7 +644,8 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
         // TM = 4: wave w owns block w of the tile; TM = 2: waves 2p and 2p+1 each copy block p and own half of it
         uint32_t blk = (tok_tile_of(ix_item) * OH_TOK_ITEM + wave * (TM * 16)) / 64;
         if (blk > last_block) blk = last_block;  // clamp: results of such tokens are never stored
-        ix_base = idx + (size_t)blk * idx_row_bytes * 64;
+        const uint32_t op = ep.op_col_tiles ? col_of(ix_item) / ep.op_col_tiles : 0u;
+        ix_base = idx + (size_t)op * ep.op_idx_stride + (size_t)blk * idx_row_bytes * 64;
         ix_lane_off = lane * 4;
     };
     // real = false (past the end of the stream): the operation re-copies the first slice of the
@@ -737,6 +743,8 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
         uint32_t je = j, ge = g;
         asm volatile("" : "+v"(je), "+v"(ge));
         const uint32_t colblk = col_of(item);
+        Epilogue epl = ep;
+        if (ep.op_col_tiles) epl.scale = scalar_load1(ep.op_scales + colblk / ep.op_col_tiles);
         const uint32_t tile_tok0 = tok_tile_of(item) * OH_TOK_ITEM;
         const uint32_t tok0 = tile_tok0 + wave * (TM * 16);
         const bool vec_store = (M % 4 == 0);
@@ -763,10 +771,10 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
                 const v4i a = acc[t][c];
                 acc[t][c] = (v4i){0, 0, 0, 0};
                 float4 o;
-                o.x = dequant<ACT>(a[0], ep, bv.x);
-                o.y = dequant<ACT>(a[1], ep, bv.y);
-                o.z = dequant<ACT>(a[2], ep, bv.z);
-                o.w = dequant<ACT>(a[3], ep, bv.w);
+                o.x = dequant<ACT>(a[0], epl, bv.x);
+                o.y = dequant<ACT>(a[1], epl, bv.y);
+                o.z = dequant<ACT>(a[2], epl, bv.z);
+                o.w = dequant<ACT>(a[3], epl, bv.w);
                 if (full) {  // workgroup-uniform: every token and column of the tile exists
                     // streaming store: the output is not read again by this kernel
                     typedef float v4f __attribute__((ext_vector_type(4)));
@@ -930,7 +938,9 @@ int launch_onehot_tm(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out,
 }
 
 // 256-token items (TM = 4) need fewer LDS reads and copies per MFMA; when the batch does not offer
-// two of them per CU, 128-token items (TM = 2) put a second wave on every SIMD instead.
+// two of them per CU, 128-token items (TM = 2) put a second wave on every SIMD instead.  In between the
+// item size that needs the shorter time wins: rounds of the persistent grid x the cost of an item (a
+// 256-token item takes 1.7 times as long as a 128-token one).
 template <int TN, bool P8>
 int launch_onehot(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_t* d_acc, uint32_t n,
                   const Epilogue& ep)
@@ -940,14 +950,17 @@ int launch_onehot(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, in
     // per-slice costs (barrier, first operand reads, bookkeeping) are paid half as often.  Measured 3-9 %
     // faster for 48- and 64-column tiles; 96-column tiles only have room for 24, which gained nothing.
     constexpr int GSB = (TN == 3 || (TN == 4 && !P8)) ? 32 : 16;
+    const uint64_t slots = 2ull * ctx->prop.multiProcessorCount;
+    const uint64_t items2 = (uint64_t)((n + oh_tok_item(2) - 1) / oh_tok_item(2)) * (a.g.M_pad / (16 * TN));
+    const bool small_items = items4 < slots || 10 * ((items2 + slots - 1) / slots) < 17 * ((items4 + slots - 1) / slots);
     if constexpr (GSB != 16) {
         const uint32_t entries = P8 ? a.g.CB_pad / 2 : a.g.CB_pad;
         if (entries % GSB == 0) {
-            if (items4 < 2ull * ctx->prop.multiProcessorCount) return launch_onehot_tm<TN, 2, P8, GSB>(ctx, a, d_idx, d_out, d_acc, n, ep);
+            if (small_items) return launch_onehot_tm<TN, 2, P8, GSB>(ctx, a, d_idx, d_out, d_acc, n, ep);
             return launch_onehot_tm<TN, 4, P8, GSB>(ctx, a, d_idx, d_out, d_acc, n, ep);
         }
     }
-    if (items4 < 2ull * ctx->prop.multiProcessorCount) return launch_onehot_tm<TN, 2, P8>(ctx, a, d_idx, d_out, d_acc, n, ep);
+    if (small_items) return launch_onehot_tm<TN, 2, P8>(ctx, a, d_idx, d_out, d_acc, n, ep);
     return launch_onehot_tm<TN, 4, P8>(ctx, a, d_idx, d_out, d_acc, n, ep);
 }
 
@@ -1340,6 +1353,9 @@ int launch_gather(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, in
         ep.lut_bias_term = a.desc.bias_mode == PIMDL_BIAS_TIMES_CB ? a.desc.lut_bias * (float)g.CB : a.desc.lut_bias;
         ep.bias = a.d_bias;
         ep.act = a.desc.activation;
+        ep.op_scales = a.d_op_scales;
+        ep.op_col_tiles = a.op_col_tiles;
+        ep.op_idx_stride = a.op_idx_stride;
         if (g.gather_kind == 1) {
             if (g.C_tile == 8) {
                 switch (g.q) {

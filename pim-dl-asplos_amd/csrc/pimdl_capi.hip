@@ -168,6 +168,11 @@ struct pimdl_amm_group {
     float* d_centroids;   // the members' centroids, concatenated, + derived search data
     uint32_t x_cols;      // floats per input row (one member's K)
     uint32_t max_n;
+    // Members that are matrix-core gathers of one shape also run as ONE gather launch over their column
+    // tiles side by side, into one [n][members * M] output (pimdl_amm_group_run_fused): `merged` borrows the
+    // members' geometry and owns concatenated copies of their tables, biases and scales.
+    bool has_merged;
+    Amm merged;
 };
 
 extern "C" {
@@ -295,6 +300,9 @@ int pimdl_amm_create_tuned(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const flo
     a->d_scales = nullptr;
     a->d_bias = nullptr;
     a->grouped = grouped;
+    a->d_op_scales = nullptr;
+    a->op_col_tiles = 0;
+    a->op_idx_stride = 0;
     a->nscales = grouped ? (g.CB + desc->scale_group - 1) / desc->scale_group : i8 ? 1 : 0;
     a->h_scale0 = i8 ? scales[0] : 1.0f;
 
@@ -394,16 +402,56 @@ int pimdl_amm_group_create(pimdl_ctx* ctx, pimdl_amm* const* amms, uint32_t coun
     grp->d_centroids = nullptr;
     grp->x_cols = first->g.K;
     grp->max_n = max_n;
+    grp->has_merged = false;
     rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&grp->d_centroids), ccs_centroid_bytes(g)), "hipMalloc(group centroids)");
     const size_t one = (size_t)first->g.CB * g.C * g.v;  // raw centroid floats of one member
     for (uint32_t i = 0; i < count && !rc; ++i)
         rc = hip_check(ctx, hipMemcpyAsync(grp->d_centroids + i * one, amms[i]->d_centroids, one * sizeof(float),
                                            hipMemcpyDeviceToDevice, ctx->stream), "D2D centroids");
     if (!rc) rc = launch_ccs_prep(ctx, g, grp->d_centroids);
+    // one gather launch for all members?
+    bool same = first->desc.lut_dtype == PIMDL_LUT_I8 && !first->grouped && first->g.gather_kind == 1 &&
+                first->g.M % first->g.col_block == 0;
+    const float lbt0 = first->desc.bias_mode == PIMDL_BIAS_TIMES_CB ? first->desc.lut_bias * (float)first->g.CB : first->desc.lut_bias;
+    for (uint32_t i = 1; i < count && same; ++i) {
+        const Amm* a = amms[i];
+        const float lbt = a->desc.bias_mode == PIMDL_BIAS_TIMES_CB ? a->desc.lut_bias * (float)a->g.CB : a->desc.lut_bias;
+        same = a->desc.lut_dtype == PIMDL_LUT_I8 && !a->grouped && a->g.gather_kind == 1 && a->g.M == first->g.M &&
+               a->g.q == first->g.q && a->g.C_tile == first->g.C_tile && a->g.CB_pad == first->g.CB_pad &&
+               a->lut_bytes == first->lut_bytes && a->desc.activation == first->desc.activation && lbt == lbt0;
+    }
+    if (!rc && same) {
+        Amm& m = grp->merged;
+        m = *first;  // geometry, epilogue constants; the pointers below are the group's own
+        m.d_centroids = nullptr;
+        m.d_scales = nullptr;
+        m.d_lut = nullptr;
+        m.d_bias = nullptr;
+        m.d_op_scales = nullptr;
+        m.g.M = m.g.M_pad = first->g.M * count;
+        m.desc.output_feature_len = m.g.M;
+        m.desc.max_n = max_n;
+        m.g.idx_row_bytes = g.idx_row_bytes;
+        m.op_col_tiles = first->g.M / first->g.col_block;
+        m.op_idx_stride = first->g.idx_row_bytes * 64;  // tiled index rows: a byte range is a range of 256-byte blocks
+        m.lut_bytes = first->lut_bytes * count;
+        std::vector<float> sc(count);
+        for (uint32_t i = 0; i < count; ++i) sc[i] = amms[i]->h_scale0;
+        rc = hip_check(ctx, hipMalloc(&m.d_lut, m.lut_bytes), "hipMalloc(group lut)");
+        if (!rc) rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&m.d_bias), (size_t)m.g.M * sizeof(float)), "hipMalloc(group bias)");
+        if (!rc) rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&m.d_op_scales), count * sizeof(float)), "hipMalloc(group scales)");
+        for (uint32_t i = 0; i < count && !rc; ++i) {
+            rc = hip_check(ctx, hipMemcpyAsync(static_cast<char*>(m.d_lut) + (size_t)i * first->lut_bytes, amms[i]->d_lut,
+                                               first->lut_bytes, hipMemcpyDeviceToDevice, ctx->stream), "D2D lut");
+            if (!rc) rc = hip_check(ctx, hipMemcpyAsync(m.d_bias + (size_t)i * first->g.M, amms[i]->d_bias,
+                                                        (size_t)first->g.M * sizeof(float), hipMemcpyDeviceToDevice, ctx->stream), "D2D bias");
+        }
+        if (!rc) rc = hip_check(ctx, hipMemcpy(m.d_op_scales, sc.data(), count * sizeof(float), hipMemcpyHostToDevice), "H2D group scales");
+        grp->has_merged = !rc;
+    }
     if (!rc) rc = hip_check(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
     if (rc) {
-        (void)hipFree(grp->d_centroids);
-        delete grp;
+        pimdl_amm_group_destroy(grp);
         return rc;
     }
     *out = grp;
@@ -416,8 +464,39 @@ int pimdl_amm_group_destroy(pimdl_amm_group* grp)
     (void)hipSetDevice(grp->ctx->device);
     (void)hipStreamSynchronize(grp->ctx->stream);
     (void)hipFree(grp->d_centroids);
+    if (grp->merged.d_lut) (void)hipFree(grp->merged.d_lut);
+    if (grp->merged.d_bias) (void)hipFree(grp->merged.d_bias);
+    if (grp->merged.d_op_scales) (void)hipFree(grp->merged.d_op_scales);
     delete grp;
     return PIMDL_OK;
+}
+
+int pimdl_amm_group_fused_cols(const pimdl_amm_group* grp, uint32_t* cols)
+{
+    if (!grp || !cols) return PIMDL_ERR_INVALID;
+    *cols = grp->has_merged ? grp->merged.g.M : 0;
+    return PIMDL_OK;
+}
+
+int pimdl_amm_group_run_fused(pimdl_amm_group* grp, const float* in, uint32_t n, float* out)
+{
+    if (!grp) return PIMDL_ERR_INVALID;
+    Ctx* ctx = grp->ctx;
+    if (!grp->has_merged)
+        return set_error(ctx, PIMDL_ERR_UNSUPPORTED, "pimdl_amm_group_run_fused: the members do not share one matrix-core gather shape");
+    if (!in || !out) return set_error(ctx, PIMDL_ERR_INVALID, "null buffer");
+    if (n > grp->max_n) return set_error(ctx, PIMDL_ERR_INVALID, "n=%u exceeds max_n=%u of this group", n, grp->max_n);
+    int rc = activate(ctx);
+    if (rc || n == 0) return rc;
+    const float* d_in;
+    float* d_out;
+    bool out_host;
+    if ((rc = stage_input(ctx, grp->members[0]->g, in, n, &d_in))) return rc;
+    if ((rc = stage_output(ctx, grp->merged.g, out, n, &d_out, &out_host))) return rc;
+    if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, idx_buffer_bytes(grp->g, n), "hipMalloc(index scratch)"))) return rc;
+    if ((rc = launch_ccs(ctx, grp->g, d_in, grp->d_centroids, ctx->d_idx, n, grp->x_cols))) return rc;
+    if ((rc = launch_gather(ctx, grp->merged, ctx->d_idx, d_out, nullptr, n))) return rc;
+    return finish_output(ctx, grp->merged.g, out, n, out_host);
 }
 
 int pimdl_amm_group_run(pimdl_amm_group* grp, const float* in, uint32_t n, float* const* outs)

@@ -230,6 +230,11 @@ class TransformerLayer:
         if self.fused_qkv:
             qkv = self._run("qkv", x, n)
             q, k, v = (qkv[:, i * p.token_dim:(i + 1) * p.token_dim] for i in range(3))
+        elif self.qkv_group is not None and self.qkv_group.fused_cols == 3 * p.token_dim:
+            # one search launch and one gather launch into [q | k | v]
+            qkv = torch.empty((n, 3 * p.token_dim), device=x.device, dtype=torch.float32)
+            self.qkv_group.run_fused_ptr(x.data_ptr(), n, qkv.data_ptr())
+            q, k, v = (qkv[:, i * p.token_dim:(i + 1) * p.token_dim] for i in range(3))
         elif self.qkv_group is not None:
             q, k, v = (torch.empty((n, p.token_dim), device=x.device, dtype=torch.float32) for _ in range(3))
             self.qkv_group.run_ptr(x.data_ptr(), n, [q.data_ptr(), k.data_ptr(), v.data_ptr()])

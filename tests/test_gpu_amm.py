@@ -268,6 +268,9 @@ def test_two_tokens_per_lane_in_the_fp32_table_gather(ctx, kind):
 @pytest.mark.parametrize("N,K,v,C,Ms,lut", [
     (300, 256, 4, 16, (96, 200, 64), "i8"),     # tiled index rows (matrix-core gather), three outputs of different widths
     (1000, 128, 4, 8, (128, 128), "i8"),        # paired gather
+    (1300, 128, 4, 8, (192, 192, 192), "i8"),   # paired gather, three members in one gather launch
+    (700, 256, 4, 16, (96, 96), "i8"),          # one gather launch, 96-column tiles
+    (2100, 128, 4, 16, (768, 768, 768), "i8"),  # the Q/K/V shape
     (257, 256, 2, 32, (100, 60), "i8"),         # 32 centroids: byte indices, row-major index rows
     (300, 256, 8, 16, (48, 80, 48), "f32"),     # fp32 tables
 ])
@@ -286,6 +289,15 @@ def test_operators_sharing_an_input_are_searched_by_one_launch(ctx, N, K, v, C, 
     outs2 = group.run(x[:77])  # a smaller batch through the same group
     for o, o2 in zip(outs, outs2):
         assert np.array_equal(o[:77], o2)
+    # one gather launch for all members where they are matrix-core gathers of one shape
+    same_shape = lut == "i8" and C <= 16 and len(set(Ms)) == 1 and Ms[0] % amms[0].geometry()["col_block"] == 0
+    assert (group.fused_cols > 0) == same_shape
+    if same_shape:
+        fused = group.run_fused(x)
+        assert np.array_equal(fused.view(np.uint32), np.concatenate(outs, axis=1).view(np.uint32))
+    else:
+        with pytest.raises(pimdl.PimdlError):
+            group.run_fused(x)
     group.close()
     for a in amms:
         a.close()
