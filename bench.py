@@ -136,7 +136,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (the path shards over tokens with no exchange; "
-              "see DESIGN.md); run with --gpus 1", file=sys.stderr)
+              "nothing to measure across GPUs); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
     import torch

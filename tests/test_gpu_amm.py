@@ -233,7 +233,7 @@ def test_scale_per_codebook_group(ctx, group, C, v, CB, M):
     """int8 LUT with one scale per `group` codebooks (an extension the reference does not have, so the
     only pin is the oracle's definition: int32 inside a group, then fp32 `tot += (float)acc_g * scale[g]`
     over groups ascending, then + bias).  Bit-exact against it, including ragged last groups, a group
-    larger than CB, 4- and 8-bit index rows; group 1 is BASELINE's per-codebook scale."""
+    larger than CB, 4- and 8-bit index rows; group 1 is one scale per codebook."""
     N, K = 300, CB * v
     x, cent, lut, bias = make_case(500 + group + C, N, K, v, C, M)
     ng = (CB + group - 1) // group

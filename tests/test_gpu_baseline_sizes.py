@@ -55,20 +55,20 @@ def run_and_check_sample(ctx, seed, N, K, v, C, M, lut_kind, sample=192):
 
 @pytest.mark.parametrize("K,M", [(768, 3072), (3072, 768)])
 def test_bert_base_ffn_pair_full_batch(env, K, M):
-    """configs[1]: N = 8192, v = 4, C = 16, int8 LUT."""
+    """The benchmark configuration: BERT-base FFN pair, N = 8192, v = 4, C = 16, int8 LUT."""
     run_and_check_sample(env[1], 11, 8192, K, 4, 16, M, "i8")
 
 
 @pytest.mark.parametrize("K,M", [(1024, 3072), (1024, 1024), (1024, 4096), (4096, 1024)])
 def test_bert_large_linears_full_batch(env, K, M):
-    """configs[2]: hidden 1024, FFN 4096, N = 8192 (fused QKV, O, FFN1, FFN2), v = 4, C = 16."""
+    """BERT-large: hidden 1024, FFN 4096, N = 8192 (fused QKV, O, FFN1, FFN2), v = 4, C = 16."""
     run_and_check_sample(env[1], 12, 8192, K, 4, 16, M, "i8", sample=128)
 
 
 @pytest.mark.parametrize("lut_kind", ["i8", "f32"])
 @pytest.mark.parametrize("v,C", [(2, 8), (2, 16), (2, 32), (4, 8), (4, 16), (4, 32), (8, 8), (8, 16), (8, 32)])
 def test_vit_base_sweep_full_batch(env, v, C, lut_kind):
-    """configs[3]: N = 64 x 197 = 12608, FFN1 of ViT-Base (768 -> 3072), v x C sweep, both LUT types."""
+    """ViT-Base: N = 64 x 197 = 12608, FFN1 of ViT-Base (768 -> 3072), v x C sweep, both LUT types."""
     run_and_check_sample(env[1], 13 + v + C, 12608, 768, v, C, 3072, lut_kind, sample=96)
 
 
