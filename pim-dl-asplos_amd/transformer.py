@@ -359,35 +359,53 @@ def synth_layers(params, ctx, pimdl, seed=0, shared_qkv_centroids=False):
 
 
 def main(argv=None):
-    """Counterpart of the reference's test_transformer driver:
-        python transformer.py config.yaml [weights.npz] [--iters K] [--graph]
-    reads the same YAML and weight file, runs the model forward on random token features and prints
-    the per-iteration time in the reference's wording (test_transformer.cpp:356).  --graph records the
-    forward once into a HIP graph and times its replays (no host work between the kernels)."""
-    argv = list(sys.argv[1:] if argv is None else argv)
-    iters = 5
-    use_graph = "--graph" in argv
-    if use_graph:
-        argv.remove("--graph")
-    if "--iters" in argv:
-        i = argv.index("--iters")
-        iters = int(argv[i + 1])
-        del argv[i:i + 2]
-    if not argv:
-        print("usage: transformer.py config_yaml_path [weight_path] [--iters K] [--graph]", file=sys.stderr)
+    """Counterpart of the reference's drivers (test_transformer.cpp, test_transformer_layer.cpp and the
+    run_model.py / run_layer.py scripts that call them):
+        python transformer.py config.yaml [weights.npz] [--iters K] [--graph] [--layer]
+        python transformer.py --transformer_config_file config.yaml [--model_weight_file weights.npz] ...
+    reads the same YAML and weight file, runs the forward on random token features and prints the
+    per-iteration and average time in the reference's wording (test_transformer.cpp:356,381).
+      --graph           record the forward once into a HIP graph and time its replays
+      --layer           one layer only (run_layer.py); --need_breakdown adds the time of each stage of it
+    The scripts' other flags are accepted and have nothing to do here: --need_compile (the kernels are in the
+    library), --need_measure_energy, --breakdown_type."""
+    import argparse
+    ap = argparse.ArgumentParser(prog="transformer.py")
+    ap.add_argument("config", nargs="?")
+    ap.add_argument("weights", nargs="?")
+    ap.add_argument("--transformer_config_file")          # run_model.py:8 / run_layer.py:8
+    ap.add_argument("--model_weight_file", default=None)  # run_model.py:9
+    ap.add_argument("--need_compile", action="store_true")
+    ap.add_argument("--need_measure_energy", action="store_true")
+    ap.add_argument("--need_breakdown", action="store_true")
+    ap.add_argument("--breakdown_type", type=int, default=0)
+    ap.add_argument("--iters", type=int, default=5)
+    ap.add_argument("--graph", action="store_true")
+    ap.add_argument("--layer", action="store_true")
+    try:
+        args = ap.parse_args(list(sys.argv[1:] if argv is None else argv))
+    except SystemExit:
         return 2
+    config = args.transformer_config_file or args.config
+    weights = args.model_weight_file if args.model_weight_file not in (None, "null") else args.weights
+    if not config:
+        print("usage: transformer.py config_yaml_path [weight_path] [--iters K] [--graph] [--layer]", file=sys.stderr)
+        return 2
+    iters, use_graph = args.iters, args.graph
     here = os.path.dirname(os.path.abspath(__file__))
     sys.path.insert(0, os.path.dirname(here))
     from __graft_entry__ import load_package
     pimdl = load_package()
     import torch
-    params = TransformerParams.from_yaml(argv[0])
+    params = TransformerParams.from_yaml(config)
+    if args.layer:
+        params.layer_num = 1
     print("finish parameter parsing")
     ctx = pimdl.Context(0)
     ctx.set_stream(torch.cuda.current_stream().cuda_stream)
-    if len(argv) > 1 and os.path.exists(argv[1]):
+    if weights and os.path.exists(weights):
         print("weight file is found, load weights from file.")
-        layers = load_npz(argv[1], params)
+        layers = load_npz(weights, params)
     else:
         print("weight file is not found, generate weights randomly.")
         layers = synth_layers(params, ctx, pimdl)
@@ -397,6 +415,7 @@ def main(argv=None):
     if use_graph:
         graph, static_x, _static_y = model.capture(x)
     print("inference start")
+    total = 0.0
     for i in range(iters):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -406,8 +425,41 @@ def main(argv=None):
         else:
             model.forward(x)
         torch.cuda.synchronize()
-        print(f"iteration {i}, inference time {time.perf_counter() - t0:.6f}")
+        dt = time.perf_counter() - t0
+        total += dt
+        print(f"iteration {i}, inference time {dt:.6f}")
     print("inference end")
+    if iters:
+        print(f"{iters} rounds' average inference time {total / iters:.6f}")
+    if args.need_breakdown:
+        # stage times of the first layer (device time between events, each stage launched on its own)
+        layer, keep = model.layers[0], {}
+        layer.forward(x, keep)
+        n = x.shape[0]
+
+        def timed(fn):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            fn()
+            e0.record()
+            for _ in range(10):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / 10 * 1e-3
+
+        stages = []
+        if "qkv" in layer.amm:
+            stages.append(("qkv", lambda: layer._run("qkv", x, n)))
+        else:
+            stages += [(nm, (lambda nm=nm: layer._run(nm, x, n))) for nm in ("q", "k", "v")]
+        stages += [("o", lambda: layer._run("o", keep["attn"], n)),
+                   ("attention_norm", lambda: layer._norm_residual("attention_norm", keep["o"], x)),
+                   ("ffn1", lambda: layer._run("ffn1", keep["h"], n)),
+                   ("ffn2", lambda: layer._run("ffn2", keep["gelu"], n)),
+                   ("ffn_norm", lambda: layer._norm_residual("ffn_norm", keep["ffn2"], keep["h"]))]
+        print("layer 0 breakdown (seconds):")
+        for name, fn in stages:
+            print(f"  {name:16s} {timed(fn):.6f}")
     model.close()
     ctx.close()
     return 0

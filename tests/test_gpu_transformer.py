@@ -241,6 +241,12 @@ def test_driver_prints_the_reference_wording(capsys):
     assert "iteration 1, inference time" in out and "inference end" in out
     assert T.main([CFG, "--iters", "2", "--graph"]) == 0  # the same through a recorded HIP graph
     assert "iteration 1, inference time" in capsys.readouterr().out
+    # the flag names of the reference's run_model.py / run_layer.py
+    assert T.main(["--transformer_config_file", CFG, "--model_weight_file", "null", "--need_compile", "--layer",
+                   "--need_breakdown", "--iters", "3"]) == 0
+    out = capsys.readouterr().out
+    assert "3 rounds' average inference time" in out and "ffn_norm" in out
+    assert T.main([]) == 2
 
 
 def test_column_tile_hint_and_measured_tile_search(ctx, tmp_path):
