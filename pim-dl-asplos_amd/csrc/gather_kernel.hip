@@ -1200,18 +1200,50 @@ int launch_f32_impl(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, 
     return hip_check(ctx, hipGetLastError(), "gather_f32_kernel launch");
 }
 
+// workgroups of gather_f32_kernel that one CU holds at a time (asked once per variant)
+template <int C_T, int Q, int GS, int IDX_BITS, bool GROUPED, int TPL>
+int f32_wgs_per_cu()
+{
+    static int cached = 0;
+    if (cached == 0) {
+        constexpr int LDS = 2 * GS * C_T * (f32_lut_chunked(C_T, Q) ? 16 * Q : 16 * Q + 16);
+        int q = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&q, gather_f32_kernel<C_T, Q, GS, IDX_BITS, GROUPED, TPL>, GF_THREADS,
+                                                         LDS) != hipSuccess || q < 1) {
+            (void)hipGetLastError();
+            q = 1;
+        }
+        cached = q;
+    }
+    return cached;
+}
+
+template <int C_T, int Q, int GS, int IDX_BITS, bool GROUPED>
+int launch_f32_tpl(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, uint32_t n)
+{
+    // Two tokens per lane halve the table traffic from L2 for batches that still give every CU two workgroups.
+    // The grid is not persistent, so a batch pays for whole rounds of resident workgroups, and workgroups of
+    // two tokens per lane are twice as long: for tables beyond the caches (where the ViT-Base sweep at
+    // N = 12608 measured it to matter: 5 of 6 shapes 10-28 % faster, one 7 % slower) the variant with the
+    // shorter rounds x length is taken, one token per lane counted 6 % dearer per token for its extra staging.
+    const uint64_t cus = ctx->prop.multiProcessorCount, colblocks = a.g.M_pad / (4 * Q);
+    const uint64_t wgs2 = (uint64_t)((n + 2 * GF_THREADS - 1) / (2 * GF_THREADS)) * colblocks;
+    bool two = wgs2 >= 2 * cus;
+    if (two && a.lut_bytes > (64ull << 20)) {
+        const uint64_t wgs1 = (uint64_t)((n + GF_THREADS - 1) / GF_THREADS) * colblocks;
+        const uint64_t slots1 = cus * (uint64_t)f32_wgs_per_cu<C_T, Q, GS, IDX_BITS, GROUPED, 1>();
+        const uint64_t slots2 = cus * (uint64_t)f32_wgs_per_cu<C_T, Q, GS, IDX_BITS, GROUPED, 2>();
+        two = 200 * ((wgs2 + slots2 - 1) / slots2) <= 106 * ((wgs1 + slots1 - 1) / slots1);
+    }
+    if (two) return launch_f32_impl<C_T, Q, GS, IDX_BITS, GROUPED, 2>(ctx, a, d_idx, d_out, n);
+    return launch_f32_impl<C_T, Q, GS, IDX_BITS, GROUPED, 1>(ctx, a, d_idx, d_out, n);
+}
+
 template <int C_T, int Q, int GS, int IDX_BITS>
 int launch_f32(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, uint32_t n)
 {
-    // two tokens per lane halve the table traffic from L2; for batches that still give every CU two
-    // workgroups
-    const uint64_t wgs2 = (uint64_t)((n + 2 * GF_THREADS - 1) / (2 * GF_THREADS)) * (a.g.M_pad / (4 * Q));
-    const bool two = wgs2 >= 2ull * ctx->prop.multiProcessorCount;
-    if (a.grouped)
-        return two ? launch_f32_impl<C_T, Q, GS, IDX_BITS, true, 2>(ctx, a, d_idx, d_out, n)
-                   : launch_f32_impl<C_T, Q, GS, IDX_BITS, true, 1>(ctx, a, d_idx, d_out, n);
-    return two ? launch_f32_impl<C_T, Q, GS, IDX_BITS, false, 2>(ctx, a, d_idx, d_out, n)
-               : launch_f32_impl<C_T, Q, GS, IDX_BITS, false, 1>(ctx, a, d_idx, d_out, n);
+    return a.grouped ? launch_f32_tpl<C_T, Q, GS, IDX_BITS, true>(ctx, a, d_idx, d_out, n)
+                     : launch_f32_tpl<C_T, Q, GS, IDX_BITS, false>(ctx, a, d_idx, d_out, n);
 }
 
 }  // namespace
