@@ -984,7 +984,8 @@ __global__ __launch_bounds__(GF_THREADS) void gather_f32_kernel(const uint8_t* _
                                                                uint32_t idx_row_bytes,
                                                                const float* __restrict__ bias,
                                                                const float* __restrict__ scales,
-                                                               uint32_t CB, uint32_t group, uint32_t act)
+                                                               uint32_t CB, uint32_t group, uint32_t act,
+                                                               uint32_t n_token_tiles, uint32_t by_xcd)
 {
     constexpr int FB = 4 * Q;             // columns per row
     // 32 rows of 16-byte pieces cover the 64 banks twice: two lanes of a ds_read_b128 pass that want
@@ -1006,9 +1007,15 @@ __global__ __launch_bounds__(GF_THREADS) void gather_f32_kernel(const uint8_t* _
     // TPL tokens per lane: the staged slice serves TPL * 256 tokens, so the table is streamed from L2
     // 1/TPL as often
     uint32_t tok[TPL];
+    // Workgroup p of the 1-D grid: column block p / n_token_tiles, token tile p % n_token_tiles -- or, by_xcd
+    // (column blocks a multiple of 8): workgroups go to the 8 XCDs round-robin, and XCD p % 8 takes every token
+    // tile of the column blocks congruent to it, so that a column block's part of the table is streamed
+    // through one L2 instead of all eight.
+    const uint32_t pq = by_xcd ? blockIdx.x / 8 : blockIdx.x;
+    const uint32_t tile = pq % n_token_tiles;
+    const uint32_t colblk = by_xcd ? blockIdx.x % 8 + 8 * (pq / n_token_tiles) : pq / n_token_tiles;
 #pragma unroll
-    for (int t = 0; t < TPL; ++t) tok[t] = (blockIdx.x * TPL + t) * GF_THREADS + threadIdx.x;
-    const uint32_t colblk = blockIdx.y;
+    for (int t = 0; t < TPL; ++t) tok[t] = (tile * TPL + t) * GF_THREADS + threadIdx.x;
     const uint32_t nslices = CB_pad / GS;
     const uint4* __restrict__ lut_blk = reinterpret_cast<const uint4*>(lut) + (size_t)colblk * CB_pad * C_T * Q;
     const uint32_t* idx_row[TPL];
@@ -1193,10 +1200,13 @@ int launch_f32_impl(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, 
         if (rc) return rc;
         attr_set = true;
     }
-    dim3 grid((n + GF_THREADS * TPL - 1) / (GF_THREADS * TPL), a.g.M_pad / (4 * Q));
-    hipLaunchKernelGGL(kern, grid, dim3(GF_THREADS), LDS, ctx->stream, d_idx,
+    const uint32_t n_token_tiles = (n + GF_THREADS * TPL - 1) / (GF_THREADS * TPL), colblocks = a.g.M_pad / (4 * Q);
+    const uint64_t wgs = (uint64_t)n_token_tiles * colblocks;
+    if (wgs > 0x7FFFFFFFull) return set_error(ctx, PIMDL_ERR_UNSUPPORTED, "gather: %llu workgroups", (unsigned long long)wgs);
+    const uint32_t by_xcd = colblocks % 8 == 0 ? 1u : 0u;
+    hipLaunchKernelGGL(kern, dim3((uint32_t)wgs), dim3(GF_THREADS), LDS, ctx->stream, d_idx,
                        reinterpret_cast<const float*>(a.d_lut), d_out, n, a.g.M, a.g.CB_pad, a.g.idx_row_bytes,
-                       a.d_bias, a.d_scales, a.g.CB, a.desc.scale_group, a.desc.activation);
+                       a.d_bias, a.d_scales, a.g.CB, a.desc.scale_group, a.desc.activation, n_token_tiles, by_xcd);
     return hip_check(ctx, hipGetLastError(), "gather_f32_kernel launch");
 }
 
