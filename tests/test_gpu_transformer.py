@@ -211,12 +211,25 @@ def test_model_is_the_chain_of_its_layers_and_reads_the_weight_file(ctx, tmp_pat
     model.close()
 
 
-def test_captured_forward_replays_like_the_eager_one(ctx):
+def _params_hd64():
+    """head_dim 64 and 32 codebooks per projection: the Q/K/V group with one gather launch, pimdl_attention and
+    the GELU epilogue are all on the path (the YAML configuration's head_dim 8 / 8 codebooks use none of them)."""
+    p = T.TransformerParams(16, 3, 2, 64, 128, 384, 2)
+    for op, (cb, k_in, m_out) in {"q": (32, 128, 128), "k": (32, 128, 128), "v": (32, 128, 128), "o": (32, 128, 128),
+                                  "ffn1": (32, 128, 384), "ffn2": (96, 384, 128)}.items():
+        p.shapes[op] = T.AmmShape(cb, 16, k_in, m_out)
+    return p
+
+
+@pytest.mark.parametrize("which", ["yaml", "hd64"])
+def test_captured_forward_replays_like_the_eager_one(ctx, which):
     """The model forward recorded into a HIP graph: every replay, with eager work and synchronisations
     in between and with new input copied into the static buffer, equals the eager result bit for bit."""
     import torch
-    p = T.TransformerParams.from_yaml(CFG)
+    p = T.TransformerParams.from_yaml(CFG) if which == "yaml" else _params_hd64()
     model = T.Transformer(ctx, pimdl, T.synth_layers(p, ctx, pimdl, seed=9), p)
+    if which == "hd64":
+        assert model.layers[0].qkv_group is not None
     gen = torch.Generator(device="cuda").manual_seed(4)
     xs = [torch.randn((p.n, p.token_dim), device="cuda", generator=gen) for _ in range(3)]
     want = [model.forward(x).clone() for x in xs]
