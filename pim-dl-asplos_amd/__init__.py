@@ -391,6 +391,12 @@ class Amm:
         self.ctx._check(lib().pimdl_amm_run_tiled(self._h, _ptr(x), n, _ptr(out), ctypes.byref(til)))
         return out
 
+    def run_tiled_ptr(self, in_ptr, n, out_ptr, n_stile=0, cb_mtile=0, f_stile=0, f_mtile=0):
+        """Raw addresses (device or host); output in the reference's DPU order."""
+        til = Tiling(n_stile, cb_mtile, f_stile, f_mtile)
+        self.ctx._check(lib().pimdl_amm_run_tiled(self._h, ctypes.c_void_p(in_ptr), n, ctypes.c_void_p(out_ptr),
+                                                  ctypes.byref(til)))
+
     def lut_gather_tiled(self, idx_flat, n, n_stile=0, cb_mtile=0, f_stile=0, f_mtile=0):
         idx_flat = np.ascontiguousarray(idx_flat, np.uint16).reshape(-1)
         out = np.empty(n * self.M, np.float32)

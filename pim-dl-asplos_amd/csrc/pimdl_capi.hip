@@ -44,19 +44,32 @@ static bool is_device_ptr(const void* p)
     return attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged;
 }
 
+// Grow-only scratch.  A buffer that is too small is replaced by a larger one; the old one stays allocated until
+// the context is destroyed, because a HIP graph captured from earlier calls on this context holds its address
+// (both kernels of a captured AMM were given the same buffer, so a replay stays consistent with itself).
+// While the stream is being captured nothing may be allocated: the call is refused instead.
 template <typename T>
 static int ensure(Ctx* ctx, T** buf, size_t* have, size_t need, const char* what)
 {
     if (*have >= need) return PIMDL_OK;
-    if (*buf) {
-        int rc = hip_check(ctx, hipStreamSynchronize(ctx->stream), "sync before scratch regrow");
-        if (rc) return rc;
-        (void)hipFree(*buf);
-        *buf = nullptr;
-        *have = 0;
-    }
-    int rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(buf), need), what);
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(ctx->stream, &cap) != hipSuccess) (void)hipGetLastError();
+    if (cap != hipStreamCaptureStatusNone)
+        return set_error(ctx, PIMDL_ERR_INVALID,
+                         "%s: the stream is being captured and the context's scratch (%zu bytes) would have to grow to "
+                         "%zu: run the call once outside the capture first", what, *have, need);
+    void* fresh = nullptr;
+    int rc = hip_check(ctx, hipMalloc(&fresh, need), what);
     if (rc) return rc;
+    if (*buf) {
+        try {
+            ctx->retired.push_back(*buf);
+        } catch (...) {
+            (void)hipFree(fresh);
+            return set_error(ctx, PIMDL_ERR_NOMEM, "%s: out of host memory", what);
+        }
+    }
+    *buf = static_cast<T*>(fresh);
     *have = need;
     return PIMDL_OK;
 }
@@ -233,6 +246,7 @@ int pimdl_destroy(pimdl_ctx* ctx)
     (void)hipFree(ctx->d_idx16);
     (void)hipFree(ctx->d_tmp);
     (void)hipFree(ctx->d_cent);
+    for (void* p : ctx->retired) (void)hipFree(p);
     for (auto& ev : ctx->ev)
         if (ev) (void)hipEventDestroy(ev);
     if (ctx->own_stream) (void)hipStreamDestroy(ctx->own_stream);
@@ -343,6 +357,8 @@ int pimdl_amm_create_tuned(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const flo
         else rc = hip_check(ctx, hipMemset(a->d_bias, 0, (size_t)g.M * sizeof(float)), "memset bias");
     }
     if (!rc && a->nscales) rc = hip_check(ctx, hipMemcpy(a->d_scales, scales, sizeof(float) * a->nscales, hipMemcpyHostToDevice), "H2D scales");
+    // the index scratch of the largest batch now, so that runs on device buffers never allocate
+    if (!rc) rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, idx_buffer_bytes(g, desc->max_n), "hipMalloc(index scratch)");
     if (rc) {
         pimdl_amm_destroy(a);
         return rc;
@@ -409,6 +425,7 @@ int pimdl_amm_group_create(pimdl_ctx* ctx, pimdl_amm* const* amms, uint32_t coun
         rc = hip_check(ctx, hipMemcpyAsync(grp->d_centroids + i * one, amms[i]->d_centroids, one * sizeof(float),
                                            hipMemcpyDeviceToDevice, ctx->stream), "D2D centroids");
     if (!rc) rc = launch_ccs_prep(ctx, g, grp->d_centroids);
+    if (!rc) rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, idx_buffer_bytes(g, max_n), "hipMalloc(index scratch)");
     // one gather launch for all members?
     bool same = first->desc.lut_dtype == PIMDL_LUT_I8 && !first->grouped && first->g.gather_kind == 1 &&
                 first->g.M % first->g.col_block == 0;

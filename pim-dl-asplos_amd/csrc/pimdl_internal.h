@@ -4,6 +4,7 @@
 #include <stdint.h>
 
 #include <string>
+#include <vector>
 
 #include "pimdl.h"
 
@@ -85,7 +86,9 @@ struct Ctx {
     hipStream_t stream;
     hipDeviceProp_t prop;
     std::string err;
-    // grow-only device scratch
+    // Grow-only device scratch.  A buffer that has to grow is replaced, and the old one is kept until the
+    // context is destroyed (`retired`): a HIP graph captured from earlier calls holds its address.
+    std::vector<void*> retired;
     float* d_in;
     size_t in_bytes;
     float* d_out;

@@ -81,3 +81,97 @@ def test_reference_single_amm_search_space_shape(env):
     """The shape of the reference's 89 single-AMM tuning configs: N = 32768, 1024 -> 4096, 256 codebooks of
     16 centroids (512 MB of fp32 output, 128 token tiles x 64 column tiles)."""
     run_and_check_sample(env[1], 41, 32768, 1024, 4, 16, 4096, "i8", sample=64)
+
+
+def _layer_sample_rows(rng, n, count):
+    rows = np.sort(rng.choice(n, size=count, replace=False))
+    rows[0], rows[-1] = 0, n - 1
+    return rows
+
+
+def test_bert_large_layer_full_batch(env):
+    """One BERT-large encoder layer as a layer: hidden 1024, 16 heads x 64, FFN 4096, N = 8192 (64 x 128),
+    every linear a LUT-AMM with v = 4, C = 16 -- the Q/K/V group, attention over 64 x 16 heads, both
+    LayerNorms and the GELU epilogue at this shape, each stage against the oracle on sampled rows."""
+    import torch
+    from pim_dl_asplos_amd import transformer as T
+    from layer_stage_checks import check_layer_stages
+
+    pimdl, _ = env
+    ctx = pimdl.Context(0)
+    ctx.set_stream(torch.cuda.current_stream().cuda_stream)
+    p = T.TransformerParams(128, 64, 16, 64, 1024, 4096, 1)
+    for op, (k_in, m_out) in {"q": (1024, 1024), "k": (1024, 1024), "v": (1024, 1024), "o": (1024, 1024),
+                              "ffn1": (1024, 4096), "ffn2": (4096, 1024)}.items():
+        p.shapes[op] = T.AmmShape(k_in // 4, 16, k_in, m_out)
+    rng = np.random.default_rng(31)
+    w = T.synth_layers(p, ctx, pimdl, seed=31)[0]
+    for name, _ in T.NORMS:
+        w[name]["weight"] = rng.standard_normal(p.token_dim).astype(np.float32)
+        w[name]["bias"] = rng.standard_normal(p.token_dim).astype(np.float32)
+    for name, _ in T.LINEARS:
+        w[name]["bias"] = (rng.standard_normal(w[name]["bias"].shape[0]) * 0.1).astype(np.float32)
+    layer = T.TransformerLayer(ctx, pimdl, w, p)
+    assert layer.qkv_group is not None and layer.qkv_group.fused_cols == 3 * p.token_dim
+    x = torch.from_numpy(rng.standard_normal((p.n, p.token_dim)).astype(np.float32)).cuda()
+    keep = {}
+    y = layer.forward(x, keep)
+    torch.cuda.synchronize()
+    assert y.shape == (8192, 1024) and torch.isfinite(y).all()
+    check_layer_stages(w, p, x, keep, _layer_sample_rows(rng, p.n, 96), [(0, 0), (17, 5), (63, 15)])
+    # the same call again gives the same bits (nothing of the first run is left in the scratch buffers)
+    assert torch.equal(layer.forward(x), y)
+    torch.cuda.synchronize()
+    layer.close()
+    ctx.close()
+
+
+def test_bert_base_12_layer_forward_full_batch(env):
+    """The 12-layer LUT-BERT-base forward at 32 x 128 tokens (hidden 768, 12 heads, FFN 3072, v = 4, C = 16):
+    the first and the last layer stage by stage against the oracle on sampled rows (the last one on the input
+    the eleven layers before it produced), every layer's output finite, the model equal to the chain of its
+    layers, and replays of the recorded HIP graph equal to the eager forward bit for bit."""
+    import torch
+    from pim_dl_asplos_amd import transformer as T
+    from layer_stage_checks import check_layer_stages
+
+    pimdl, _ = env
+    ctx = pimdl.Context(0)
+    ctx.set_stream(torch.cuda.current_stream().cuda_stream)
+    p = T.TransformerParams.bert_base(batch_size=32, seq_len=128, layer_num=12)
+    layers = T.synth_layers(p, ctx, pimdl, seed=32)
+    model = T.Transformer(ctx, pimdl, layers, p)
+    rng = np.random.default_rng(32)
+    # token ids uniform over a 30522-word vocabulary, features = word + position embedding (random-init; the
+    # reference has no embedding layer, its driver feeds random features)
+    ids = torch.from_numpy(rng.integers(0, 30522, p.n)).cuda()
+    gen = torch.Generator(device="cuda").manual_seed(32)
+    word = torch.randn((30522, p.token_dim), device="cuda", generator=gen) * 0.02
+    pos = torch.randn((p.seq_len, p.token_dim), device="cuda", generator=gen) * 0.02
+    x = (word[ids] + pos.repeat(p.batch_size, 1)).contiguous()
+    # layer by layer, keeping the intermediates of the first and the last layer
+    z, keeps, inputs = x, {}, {}
+    for li, layer in enumerate(model.layers):
+        keep = {} if li in (0, 11) else None
+        if keep is not None:
+            inputs[li], keeps[li] = z, keep
+        z = layer.forward(z, keep)
+        assert torch.isfinite(z).all(), f"layer {li}"
+    torch.cuda.synchronize()
+    for li in (0, 11):
+        check_layer_stages(layers[li], p, inputs[li], keeps[li], _layer_sample_rows(rng, p.n, 64), [(0, 0), (31, 11)])
+    y = model.forward(x)
+    assert torch.equal(y, z)
+    graph, static_x, static_y = model.capture(x)
+    x2 = (word[ids.flip(0)] + pos.repeat(p.batch_size, 1)).contiguous()
+    y2 = model.forward(x2).clone()
+    for xin, want in ((x, y), (x2, y2), (x, y)):
+        static_x.copy_(xin)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_y, want)
+        assert torch.equal(model.forward(x2), y2)  # eager work between the replays, same context
+        torch.cuda.synchronize()
+    del graph
+    model.close()
+    ctx.close()

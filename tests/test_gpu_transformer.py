@@ -247,6 +247,68 @@ def test_captured_forward_replays_like_the_eager_one(ctx, which):
     model.close()
 
 
+def test_graph_survives_growth_of_the_context_scratch():
+    """A recorded graph holds the addresses of the context's scratch buffers.  Later eager calls that need more
+    scratch (a larger operator, a larger batch, host buffers, the debug outputs) must leave those addresses
+    valid: the replay after them still equals the eager result."""
+    import torch
+    c = pimdl.Context(0)
+    c.set_stream(torch.cuda.current_stream().cuda_stream)
+    p = _params_hd64()
+    model = T.Transformer(c, pimdl, T.synth_layers(p, c, pimdl, seed=10), p)
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn((p.n, p.token_dim), device="cuda", generator=gen)
+    want = model.forward(x).clone()
+    graph, static_x, static_y = model.capture(x)
+    # everything that makes the scratch grow: 4096 tokens x 768 codebooks against 48 tokens x 96 before
+    rng = np.random.default_rng(3)
+    N, K, v, C, M = 4096, 3072, 4, 16, 256
+    cent = rng.standard_normal((K // v, C, v)).astype(np.float32)
+    lut = rng.integers(-128, 128, (K // v, C, M)).astype(np.int8)
+    big = c.amm(cent, lut, np.float32(0.01), None, max_n=N)
+    xb = rng.standard_normal((N, K)).astype(np.float32)
+    out_host, idx, acc = big.run_debug(xb)                      # host staging, index and accumulator scratch
+    xd = torch.from_numpy(xb).cuda()
+    od = torch.empty((N, M), device="cuda")
+    big.run_ptr(xd.data_ptr(), N, od.data_ptr())                # device buffers
+    torch.cuda.synchronize()
+    assert np.array_equal(od.cpu().numpy().view(np.uint32), out_host.view(np.uint32))
+    for _ in range(2):
+        static_x.copy_(x)
+        static_y.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_y, want)
+    # during a capture the scratch cannot grow: the call is refused, not served from a fresh allocation
+    huge = c.amm(cent, lut, np.float32(0.01), None, max_n=N)
+    ot = torch.empty((N, M), device="cuda")
+    g2 = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    c.set_stream(side.cuda_stream)
+    refused = None
+    try:
+        with torch.cuda.graph(g2, stream=side, capture_error_mode="thread_local"):
+            try:  # a tiled run needs a row-major staging buffer that no call has sized yet
+                huge.run_tiled_ptr(xd.data_ptr(), N, ot.data_ptr(), n_stile=1024, f_stile=128)
+            except pimdl.PimdlError as e:
+                refused = e
+    finally:
+        c.set_stream(torch.cuda.current_stream().cuda_stream)
+    assert refused is not None and refused.code == pimdl.ERR_INVALID and "captured" in str(refused)
+    # outside the capture the same call is served, and equals the row-major result re-ordered
+    huge.run_tiled_ptr(xd.data_ptr(), N, ot.data_ptr(), n_stile=1024, f_stile=128)
+    torch.cuda.synchronize()
+    tiled = ot.cpu().numpy().reshape(-1)
+    for n_, f_ in zip(rng.integers(0, N, 200), rng.integers(0, M, 200)):
+        assert tiled[oracle.output_offset(int(n_), int(f_), 1024, 128, 128, M // 128)] == out_host[n_, f_]
+    del graph, g2
+    big.close()
+    huge.close()
+    model.close()
+    c.close()
+
+
 def test_driver_prints_the_reference_wording(capsys):
     assert T.main([CFG, "--iters", "2"]) == 0
     out = capsys.readouterr().out
