@@ -138,6 +138,20 @@ PIMDL_API int pimdl_amm_destroy(pimdl_amm* amm);
  * stream and the call returns at once; use pimdl_synchronize() or stream ordering. */
 PIMDL_API int pimdl_amm_run(pimdl_amm* amm, const float* in, uint32_t n, float* out);
 
+/* pimdl_amm_run for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  It calls no hipMalloc, hipFree
+ * or other allocating routine: the packed centroid indices that travel from the search kernel to the gather
+ * kernel live in a fixed array of PIMDL_NOALLOC_SCRATCH_BYTES inside the library's device image (each GPU
+ * the library runs on holds its copy until the process ends) instead of the context's grow-only scratch.
+ *   in_dev, out_dev  DEVICE pointers, fp32 [n][K] and [n][M]; queued on the context's stream, returns at once.
+ *   PIMDL_ERR_INVALID when a pointer is a host pointer, or when n tokens need more index bytes than the array
+ *   holds: n rounded up to 64, times num_codebook rounded up to 32, times 1/2 byte (up to 16 centroids) or
+ *   1 byte (more).  BERT-base's 3072 -> 768 matrix at n = 8192 needs 3 MiB.
+ * Output bits are those of pimdl_amm_run.  Every call on one GPU, from any context or thread, shares that
+ * GPU's array: calls that overlap in time on one GPU race (calls queued on one stream do not overlap). */
+#define PIMDL_NOALLOC_SCRATCH_BYTES (8u << 20)
+PIMDL_API int pimdl_amm_run_noalloc(pimdl_amm* amm, const float* in_dev, uint32_t n, float* out_dev);
+
 /* As pimdl_amm_run, plus the two intermediates that make the bit-exact claims checkable:
  *   idx_out  host uint16 [n][CB] centroid ids (what index_calculation writes under the
  *            identity tiling, src/host/index_calc_host.cpp:41-49), or NULL

@@ -31,7 +31,8 @@ EXPORTS = ["pimdl_init", "pimdl_destroy", "pimdl_last_error", "pimdl_set_stream"
            "pimdl_amm_run_tiled", "pimdl_lut_gather_tiled", "pimdl_lutgen",
            "pimdl_layer_norm", "pimdl_get_device_info", "pimdl_amm_get_geometry", "pimdl_diag_bandwidth",
            "pimdl_diag_mfma_error", "pimdl_amm_group_create", "pimdl_amm_group_run", "pimdl_amm_group_destroy",
-           "pimdl_attention", "pimdl_amm_group_fused_cols", "pimdl_amm_group_run_fused"]
+           "pimdl_attention", "pimdl_amm_group_fused_cols", "pimdl_amm_group_run_fused", "pimdl_amm_run_noalloc"]
+NOALLOC_SCRATCH_BYTES = 8 << 20
 
 
 class PimdlError(RuntimeError):
@@ -116,6 +117,7 @@ def lib():
     L.pimdl_amm_create_tuned.argtypes = [vp, ctypes.POINTER(AmmDesc), vp, vp, vp, vp, u32, ctypes.POINTER(vp)]
     L.pimdl_amm_destroy.argtypes = [vp]
     L.pimdl_amm_run.argtypes = [vp, vp, u32, vp]
+    L.pimdl_amm_run_noalloc.argtypes = [vp, vp, u32, vp]
     L.pimdl_amm_run_debug.argtypes = [vp, vp, u32, vp, vp, vp]
     L.pimdl_amm_profile.argtypes = [vp, vp, u32, vp, u32, u32, ctypes.POINTER(AmmTiming)]
     L.pimdl_index_calculation.argtypes = [vp, vp, vp, u32, u32, u32, u32, vp, u32, u32]
@@ -357,6 +359,10 @@ class Amm:
     def run_ptr(self, in_ptr, n, out_ptr):
         """Raw addresses (device or host), e.g. torch tensors' data_ptr(); asynchronous for device memory."""
         self.ctx._check(lib().pimdl_amm_run(self._h, ctypes.c_void_p(in_ptr), n, ctypes.c_void_p(out_ptr)))
+
+    def run_noalloc_ptr(self, in_ptr, n, out_ptr):
+        """Device addresses only; the call allocates nothing (fixed scratch inside the library)."""
+        self.ctx._check(lib().pimdl_amm_run_noalloc(self._h, ctypes.c_void_p(in_ptr), n, ctypes.c_void_p(out_ptr)))
 
     def run_debug(self, x, want_acc=True):
         x = np.ascontiguousarray(x, np.float32)

@@ -5,13 +5,41 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
 #include <vector>
 
 #include "pimdl_internal.h"
 
+// Scratch of pimdl_amm_run_noalloc: the packed centroid indices that the search kernel writes and the gather
+// kernel reads.  A file-scope device array, so the entry point never allocates; every GPU the library runs on
+// holds its own copy until the process ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress: kernels and memory calls get the device address that call returned (kept per device in
+// g_scratch_ptr, and per context in Ctx::d_static_scratch).
+static __device__ __align__(256) unsigned char scratch[PIMDL_NOALLOC_SCRATCH_BYTES];
+
 namespace pimdl {
 
 static thread_local std::string g_init_error;
+
+constexpr int MAX_DEVICES = 64;
+static std::mutex g_scratch_mutex;
+static unsigned char* g_scratch_ptr[MAX_DEVICES];  // device address of `scratch` on each device, once asked for
+
+// Address of this device's copy of `scratch` (the device must be current).
+static int static_scratch_address(Ctx* ctx, int device, unsigned char** out)
+{
+    if (device < 0 || device >= MAX_DEVICES) return set_error(ctx, PIMDL_ERR_UNSUPPORTED, "device %d: at most %d devices", device, MAX_DEVICES);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[device]) {
+        unsigned char* p = nullptr;
+        int rc = hip_check(ctx, hipGetSymbolAddress(reinterpret_cast<void**>(&p), HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)");
+        if (rc) return rc;
+        if (!p) return set_error(ctx, PIMDL_ERR_HIP, "hipGetSymbolAddress(scratch) returned a null address");
+        g_scratch_ptr[device] = p;
+    }
+    *out = g_scratch_ptr[device];
+    return PIMDL_OK;
+}
 
 int set_error(Ctx* ctx, int code, const char* fmt, ...)
 {
@@ -215,8 +243,10 @@ int pimdl_init(int device, pimdl_ctx** out)
     ctx->d_idx16 = nullptr; ctx->idx16_bytes = 0;
     ctx->d_tmp = nullptr; ctx->tmp_bytes = 0;
     ctx->d_cent = nullptr; ctx->cent_bytes = 0;
+    ctx->d_static_scratch = nullptr;
     for (auto& ev : ctx->ev) ev = nullptr;
     int rc = hip_check(ctx, hipSetDevice(device), "hipSetDevice");
+    if (!rc) rc = static_scratch_address(ctx, device, &ctx->d_static_scratch);
     if (!rc) rc = hip_check(ctx, hipGetDeviceProperties(&ctx->prop, device), "hipGetDeviceProperties");
     if (!rc && strncmp(ctx->prop.gcnArchName, "gfx950", 6) != 0)
         rc = set_error(ctx, PIMDL_ERR_UNSUPPORTED, "pimdl_init: device %d is %s; the kernels are built for gfx950 only",
@@ -559,6 +589,27 @@ int pimdl_amm_run(pimdl_amm* a, const float* in, uint32_t n, float* out)
     if ((rc = launch_ccs(ctx, a->g, d_in, a->d_centroids, ctx->d_idx, n))) return rc;
     if ((rc = launch_gather(ctx, *a, ctx->d_idx, d_out, nullptr, n))) return rc;
     return finish_output(ctx, a->g, out, n, out_host);
+}
+
+int pimdl_amm_run_noalloc(pimdl_amm* a, const float* in_dev, uint32_t n, float* out_dev)
+{
+    int rc = check_run_args(a, in_dev, out_dev, n);
+    if (rc) return rc;
+    Ctx* ctx = a->ctx;
+    if (!is_device_ptr(in_dev) || !is_device_ptr(out_dev))
+        return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_run_noalloc: in and out must be device pointers (staging host buffers would allocate)");
+    const size_t need = idx_buffer_bytes(a->g, n);
+    if (need > (size_t)PIMDL_NOALLOC_SCRATCH_BYTES)
+        return set_error(ctx, PIMDL_ERR_INVALID,
+                         "pimdl_amm_run_noalloc: n=%u tokens x %u index bytes per token = %zu bytes of packed indices exceed the "
+                         "fixed scratch of %u bytes; use pimdl_amm_run or a smaller batch", n, a->g.idx_row_bytes, need,
+                         (unsigned)PIMDL_NOALLOC_SCRATCH_BYTES);
+    if (n == 0) return PIMDL_OK;
+    // Nothing in the scratch has to start at zero: the search kernel writes every index byte the gather reads,
+    // padded codebooks included, and index bytes of tokens past n only reach accumulators that are never stored.
+    uint8_t* d_idx = ctx->d_static_scratch;  // the device address from hipGetSymbolAddress, never the array's name
+    if ((rc = launch_ccs(ctx, a->g, in_dev, a->d_centroids, d_idx, n))) return rc;
+    return launch_gather(ctx, *a, d_idx, out_dev, nullptr, n);
 }
 
 int pimdl_amm_run_debug(pimdl_amm* a, const float* in, uint32_t n, float* out, uint16_t* idx_out, int32_t* acc_out)

@@ -89,6 +89,7 @@ struct Ctx {
     // Grow-only device scratch.  A buffer that has to grow is replaced, and the old one is kept until the
     // context is destroyed (`retired`): a HIP graph captured from earlier calls holds its address.
     std::vector<void*> retired;
+    uint8_t* d_static_scratch;  // this device's copy of the allocation-free entry point's file-scope array
     float* d_in;
     size_t in_bytes;
     float* d_out;
