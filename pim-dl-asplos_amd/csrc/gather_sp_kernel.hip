@@ -1,0 +1,477 @@
+// LUT gather-accumulate on the sparse matrix instruction (gfx950), int8 tables with 9..16 centroids.
+//
+// Same operator as the other gather kernels (inference-engine/src/dpu/pim_lut_kernel.c:97-2296, row-major
+// statement inference-engine/test/test_amm.cpp:164-175, epilogue inference-engine/src/host/pim_lut_host.cpp:190-203):
+//     acc[n][f] = sum over cb of lut[cb][idx[n][cb]][f]          (int8 table, int32 sum, exact)
+// in the reference's own matrix form (model-calibration/LUTNeuro/LUTLinear_t.py:78, bmm(one_hot, lut)).
+//
+// A one-hot row over the 16 centroids of a codebook has at most one non-zero in every group of four
+// positions, which is a valid 2:4 structured-sparse operand.  v_smfmac_i32_16x16x128_i8 multiplies a
+// 16 x 128 matrix given in that compressed form (per lane: 16 value bytes + 16 two-bit positions) by a dense
+// 128 x 16 one: with the one-hot as the sparse operand, ONE instruction gathers and adds 8 codebooks for
+// 16 tokens x 16 columns, twice what the dense v_mfma_i32_16x16x64_i8 form of the one-hot product does, at
+// the same issue rate (measured: 16.5 clocks per instruction and SIMD for either).
+//
+// Operands of one instruction (K-step = 8 codebooks b = 0..7 of a slice), lane l = 16 g + i:
+//   sparse A (tokens x K)  lane (g, i) holds, for token i of the 16-token group, codebooks 2g (value bytes
+//             0..7) and 2g+1 (value bytes 8..15): each codebook is four groups of two value slots; the group
+//             that contains the token's centroid c (group c / 4) has value 1 in its first slot with position
+//             c % 4, everything else is 0.  Both codebooks' nibbles are one byte of the packed index row.
+//             The 8 value bytes and the 16 position bits of a nibble come from a 256-byte table in LDS
+//             (entry c: 8 value bytes, position bits for the low half, position bits for the high half).
+//   dense B (K x columns)  lane (g, j) holds column j's 16 centroid entries of codebook g (bytes 0..15) and
+//             of codebook g + 4 (bytes 16..31): two 16-byte reads of the tiled table, whose layout is that
+//             of the dense one-hot kernel ([column tile][codebook][column][16 centroids]).
+//   D (tokens x columns)   lane (g, j) holds tokens 4g..4g+3 of the group for column j.
+// (This pairing of lane groups and codebooks was read off the instruction on the device with one-hot probes.)
+//
+// A lane thus ends up with four tokens of ONE column per 16-column group.  So that its stores are still
+// 16 bytes wide, the columns of a tile are dealt to the 16-column groups in pieces: the first 4 * (TN / 4)
+// groups in fours (group c of a four holds columns 4 j + c: a lane's four accumulator tiles are four
+// consecutive columns), then a pair (columns 2 j + c), then a single group.  The permutation is applied once
+// when the table is tiled at upload (sparse_tile_column); reads of the table from LDS stay consecutive.
+//
+// Work decomposition, staging through LDS with global_load_lds, the dealing of items to the XCDs, the fused
+// de-quantisation / bias / GELU epilogue and operator groups are those of the dense one-hot kernel.
+#include "gather_common.h"
+
+namespace pimdl {
+
+// column (within its tile of 16 * tn columns) stored at position s = 16 c + j of the tile
+uint32_t sparse_tile_column(uint32_t tn, uint32_t s)
+{
+    const uint32_t c = s / 16, j = s % 16;
+    const uint32_t n4 = tn / 4 * 4;                 // groups dealt in fours
+    const uint32_t n2 = n4 + (tn % 4) / 2 * 2;      // ... then a pair
+    if (c < n4) return 16 * (c / 4 * 4) + 4 * j + c % 4;
+    if (c < n2) return 16 * n4 + 2 * j + (c - n4);
+    return 16 * c + j;
+}
+
+namespace {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+
+constexpr int SP_WAVES = 4;
+constexpr int SP_THREADS = SP_WAVES * 64;
+constexpr int sp_tok_item(int tm) { return SP_WAVES * tm * 16; }
+constexpr int sp_nbuf(int gs) { return gs > 16 ? 2 : 3; }
+constexpr int SP_TABLE = 256;  // 16 entries of 16 bytes
+constexpr int sp_lds_bytes(int tn, int gs)
+{
+    return SP_TABLE + sp_nbuf(gs) * gs * 16 * tn * 16 + sp_nbuf(gs) * SP_WAVES * 64 * 4 * (gs / 8);
+}
+
+template <int OFF>
+__device__ __forceinline__ void lds_read64(v2i& dst, uint32_t addr)
+{
+    asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+template <int N>
+__device__ __forceinline__ void lgkm_wait()
+{
+    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N < 15 ? N : 15) : "memory");
+}
+
+template <int TN, int TM, int GS>
+__global__ __launch_bounds__(SP_THREADS, 2) void gather_sparse_kernel(
+    const uint8_t* __restrict__ idx, const int8_t* __restrict__ lut, float* __restrict__ out,
+    int32_t* __restrict__ acc_out, uint32_t N, uint32_t M, uint32_t CB_pad, uint32_t idx_row_bytes,
+    uint32_t n_token_tiles, uint32_t n_items, Epilogue ep, XcdMap xmap)
+{
+    constexpr int TOK_ITEM = sp_tok_item(TM);
+    static_assert(TM == 4 || TM == 2, "a wave owns a whole or half a 64-token index block");
+    constexpr int WN = 16 * TN;                    // columns per item
+    constexpr int G = GS;                          // codebooks per slice
+    constexpr int SLICE = G * WN * 16;             // bytes of one codebook slice
+    constexpr int KSTEPS = G / 8;                  // one instruction covers 8 codebooks
+    constexpr int IWORDS = G / 8;                  // 32-bit index words per token and slice (8 nibbles each)
+    constexpr int NBLK = SLICE / 1024;             // 1 KB blocks (one copy instruction of a wave) per slice
+    constexpr int DMA_PER_WAVE = (NBLK + SP_WAVES - 1) / SP_WAVES;
+    static_assert(KSTEPS >= 2, "the operand pipeline below re-arms inside a slice");
+
+    // LDS: table (256 B) | NBUF LUT slice buffers | NIBUF index buffers
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    constexpr int NBUF = sp_nbuf(GS), NIBUF = NBUF;
+    constexpr int PD = NBUF - 1;  // prefetch distance of the LUT stream, in slices
+    constexpr uint32_t BUF0 = SP_TABLE;
+    constexpr uint32_t IBUF0 = BUF0 + NBUF * SLICE;
+    constexpr uint32_t IBYTES = SP_WAVES * 64 * 4 * IWORDS;   // index bytes of one slice (a 64-token block per wave)
+    constexpr uint32_t IWAVE = 64 * 4 * IWORDS;               // ... of one wave's 64 tokens
+    constexpr int IX_OPS = IWORDS;                            // 64 lanes x 4 B = 64 tokens x 1 word
+    constexpr int DMA_OPS = DMA_PER_WAVE + IX_OPS;            // memory operations per wave and slice
+
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t j = lane & 15;  // token within a group (sparse operand) / column within a group (dense operand, result)
+    const uint32_t g = lane >> 4;
+    if (blockIdx.x >= n_items) return;  // whole workgroup
+    const uint32_t nslices = CB_pad / G;
+    const uint32_t my_items = (n_items - blockIdx.x + gridDim.x - 1) / gridDim.x;
+    const uint32_t total = my_items * nslices;
+
+    // Table entry c (16 bytes): value bytes of a codebook whose centroid is c (first slot of group c / 4 is 1),
+    // then the position bits (c % 4 at value slot 2 (c / 4), two bits per slot) as they stand in the low half
+    // of the lane's position word, then the same bits shifted to the high half.
+    if (threadIdx.x < 64) {
+        const uint32_t c = threadIdx.x >> 2, w = threadIdx.x & 3, grp = c >> 2, pos = c & 3;
+        uint32_t word;
+        if (w < 2) word = (grp >> 1) == w ? (1u << (16 * (grp & 1))) : 0u;  // value bytes 0..3 / 4..7: slot 2 grp
+        else word = (pos << (4 * grp)) << (w == 3 ? 16 : 0);
+        reinterpret_cast<uint32_t*>(smem)[threadIdx.x] = word;
+    }
+
+    auto col_of = [&](uint32_t p) { uint32_t c, t; xmap.decode(p, n_token_tiles, c, t); return c; };
+    auto tok_tile_of = [&](uint32_t p) { uint32_t c, t; xmap.decode(p, n_token_tiles, c, t); return t; };
+    uint32_t lut_item = blockIdx.x, lut_s = 0, ix_item = blockIdx.x, ix_s = 0;
+    const int8_t* dma_base;   // uniform: start of the slice at the LUT stream position
+    const uint32_t dma_lane = wave * 1024 + lane * 16;
+    const uint8_t* ix_base;   // uniform: the 256-byte block of index words at the index stream position
+    uint32_t ix_lane_off;
+    auto locate_lut = [&]() { dma_base = lut + (size_t)col_of(lut_item) * CB_pad * (WN * 16); };
+    const uint32_t last_block = (N - 1) / 64;
+    auto locate_ix = [&]() {
+        uint32_t blk = (tok_tile_of(ix_item) * TOK_ITEM + wave * (TM * 16)) / 64;
+        if (blk > last_block) blk = last_block;  // clamp: results of such tokens are never stored
+        const uint32_t op = ep.op_col_tiles ? col_of(ix_item) / ep.op_col_tiles : 0u;
+        ix_base = idx + (size_t)op * ep.op_idx_stride + (size_t)blk * idx_row_bytes * 64;
+        ix_lane_off = lane * 4;
+    };
+    // real = false (past the end of the stream): the operation re-copies the first slice of the table into a
+    // buffer nobody reads any more, so that every slice issues the same number of operations and the waits
+    // can count them
+    auto lut_op = [&](uint32_t buf, bool real, auto uc) {
+        constexpr int u = decltype(uc)::value;
+        const uint32_t dst = BUF0 + buf * SLICE + wave * 1024;
+        const uint32_t off = (wave + SP_WAVES * u < NBLK) ? SP_WAVES * u * 1024 : 0;
+        const int8_t* src = (real ? dma_base : lut) + off;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + dma_lane),
+                                         (__attribute__((address_space(3))) void*)(smem + dst + off), 16, 0, 0);
+    };
+    auto lut_advance = [&]() {
+        dma_base += SLICE;
+        if (++lut_s == nslices) {
+            lut_s = 0;
+            lut_item += gridDim.x;
+            locate_lut();  // may point past the last item; never dereferenced then
+        }
+    };
+    auto stage_lut = [&](uint32_t buf) {
+        static_for<0, DMA_PER_WAVE>([&](auto uc) { lut_op(buf, true, uc); });
+        lut_advance();
+    };
+    auto ix_op = [&](uint32_t ibuf, bool real, auto ic) {
+        constexpr int i = decltype(ic)::value;
+        const uint32_t dst = IBUF0 + ibuf * IBYTES + wave * IWAVE;
+        const uint8_t* src = real ? ix_base + 256 * i : idx;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + (real ? ix_lane_off : 0u)),
+                                         (__attribute__((address_space(3))) void*)(smem + dst + 256 * i), 4, 0, 0);
+    };
+    auto ix_advance = [&]() {
+        ix_base += IWORDS * 256;
+        if (++ix_s == nslices) {
+            ix_s = 0;
+            ix_item += gridDim.x;
+            if (ix_item < n_items) locate_ix();
+        }
+    };
+    auto stage_ix = [&](uint32_t ibuf) {
+        static_for<0, IX_OPS>([&](auto ic) { ix_op(ibuf, true, ic); });
+        ix_advance();
+    };
+    // Index word k of a token holds the nibbles of codebooks 8k .. 8k+7 of the slice; this lane's two are byte g.
+    // Stored pre-masked twice, so that one v_bfe_u32 yields nibble * 16, the table entry's offset.
+    const uint32_t byte_shift = 8 * g;
+    const uint32_t ix_lane = IBUF0 + wave * IWAVE + (((wave * (TM * 16)) & 63) + j) * 4;
+    auto read_ix = [&](uint32_t (&raw)[TM][IWORDS], uint32_t ibuf) {
+        const uint32_t addr = ix_lane + ibuf * IBYTES;
+        static_for<0, TM * IWORDS>([&](auto ec) {
+            constexpr int t = decltype(ec)::value / IWORDS, i = decltype(ec)::value % IWORDS;
+            lds_read32<(i * 64 + t * 16) * 4>(raw[t][i], addr);
+        });
+    };
+    auto unpack_ix = [&](uint32_t (&lo)[TM][IWORDS], uint32_t (&hi)[TM][IWORDS], uint32_t (&raw)[TM][IWORDS]) {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int t = 0; t < TM; ++t)
+#pragma unroll
+            for (int i = 0; i < IWORDS; ++i) asm volatile("" : "+v"(raw[t][i]));
+#pragma unroll
+        for (int t = 0; t < TM; ++t)
+#pragma unroll
+            for (int i = 0; i < IWORDS; ++i) {
+                lo[t][i] = (raw[t][i] << 4) & 0xF0F0F0F0u;
+                hi[t][i] = raw[t][i] & 0xF0F0F0F0u;
+            }
+    };
+
+    v4i acc[TM][TN];
+#pragma unroll
+    for (int t = 0; t < TM; ++t)
+#pragma unroll
+        for (int c = 0; c < TN; ++c) acc[t][c] = (v4i){0, 0, 0, 0};
+
+    // ---- epilogue ------------------------------------------------------------------------------------
+    // Lane (g, j) holds acc[t][c][r] = sum for token 16 t + 4 g + r and the column that sparse_tile_column
+    // assigns to position 16 c + j.  Pieces of W = 4, 2 or 1 groups give W consecutive columns per lane.
+    constexpr int N4 = TN / 4 * 4, N2 = N4 + (TN % 4) / 2 * 2;
+    constexpr int NPIECES = TN / 4 + (TN % 4) / 2 + TN % 2;
+    constexpr int EPI_STORES = TM * 4 * NPIECES;  // stores of a wave in the epilogue of a full tile
+    auto epilogue_as = [&](uint32_t item, auto actc) __attribute__((always_inline)) -> bool {
+        constexpr bool ACT = decltype(actc)::value;
+        uint32_t je = j, ge = g;
+        asm volatile("" : "+v"(je), "+v"(ge));  // keeps the address arithmetic below out of the slice loop
+        const uint32_t colblk = col_of(item);
+        Epilogue epl = ep;
+        if (ep.op_col_tiles) epl.scale = scalar_load1(ep.op_scales + colblk / ep.op_col_tiles);
+        const uint32_t tile_tok0 = tok_tile_of(item) * TOK_ITEM;
+        const uint32_t tok0 = tile_tok0 + wave * (TM * 16) + 4 * ge;
+        const bool vec_ok = (M % 4 == 0);
+        const bool full = vec_ok && !acc_out && tile_tok0 + TOK_ITEM <= N && (colblk + 1) * WN <= M;
+        auto piece = [&](auto c0c, auto wc) __attribute__((always_inline)) {
+            constexpr int c0 = decltype(c0c)::value, W = decltype(wc)::value;
+            const uint32_t f = colblk * WN + 16 * c0 + W * je;  // first of this lane's W columns
+            float bv[W];
+#pragma unroll
+            for (int e = 0; e < W; ++e) bv[e] = (ep.bias && f + e < M) ? ep.bias[f + e] : 0.0f;
+#pragma unroll
+            for (int t = 0; t < TM; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const uint32_t tok = tok0 + t * 16 + r;
+                    float o[W];
+                    int32_t a[W];
+#pragma unroll
+                    for (int e = 0; e < W; ++e) {
+                        a[e] = acc[t][c0 + e][r];
+                        o[e] = dequant<ACT>(a[e], epl, bv[e]);
+                    }
+                    float* dst = out + (size_t)tok * M + f;
+                    if (full) {  // workgroup-uniform: every token and column of the tile exists
+                        if constexpr (W == 4) {
+                            typedef float v4f __attribute__((ext_vector_type(4)));
+                            __builtin_nontemporal_store((v4f){o[0], o[1], o[2], o[3]}, reinterpret_cast<v4f*>(dst));
+                        } else if constexpr (W == 2) {
+                            typedef float v2f __attribute__((ext_vector_type(2)));
+                            __builtin_nontemporal_store((v2f){o[0], o[1]}, reinterpret_cast<v2f*>(dst));
+                        } else {
+                            __builtin_nontemporal_store(o[0], dst);
+                        }
+                        continue;
+                    }
+                    if (tok >= N) continue;
+#pragma unroll
+                    for (int e = 0; e < W; ++e)
+                        if (f + e < M) {
+                            dst[e] = o[e];
+                            if (acc_out) acc_out[(size_t)tok * M + f + e] = a[e];
+                        }
+                }
+        };
+        static_for<0, TN / 4>([&](auto pc) { piece(std::integral_constant<int, 4 * decltype(pc)::value>{}, std::integral_constant<int, 4>{}); });
+        if constexpr (N2 > N4) piece(std::integral_constant<int, N4>{}, std::integral_constant<int, 2>{});
+        if constexpr (TN > N2) piece(std::integral_constant<int, N2>{}, std::integral_constant<int, 1>{});
+#pragma unroll
+        for (int t = 0; t < TM; ++t)
+#pragma unroll
+            for (int c = 0; c < TN; ++c) acc[t][c] = (v4i){0, 0, 0, 0};
+        return full;
+    };
+    auto epilogue = [&](uint32_t item) __attribute__((always_inline)) -> bool {
+        return ep.act == PIMDL_ACT_GELU_TANH ? epilogue_as(item, std::true_type{}) : epilogue_as(item, std::false_type{});
+    };
+
+    // ---- prologue: slices 0 .. PD-1, index words 0 .. PD ------------------------------------------------
+    locate_lut();
+    locate_ix();
+    static_for<0, PD + 1>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        if (i < total) stage_ix(i);
+    });
+    static_for<0, PD>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        if (i < total) stage_lut(i);
+    });
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();  // also: the table is complete
+    uint32_t iw_lo[TM][IWORDS], iw_hi[TM][IWORDS], iw_raw[TM][IWORDS];
+    read_ix(iw_raw, 0);
+    unpack_ix(iw_lo, iw_hi, iw_raw);
+
+    uint32_t item0 = blockIdx.x;
+    const uint32_t b_lane = BUF0 + (g * WN + j) * 16;  // this lane's 16 bytes of codebook g, column position j
+    uint32_t buf = 0, ibuf_next = 1;
+    uint32_t k = 0;
+    bool stores_behind = false;
+    constexpr bool COUNT_STORES = (PD - 1) * DMA_OPS + EPI_STORES <= 63;  // memory counter range
+
+    for (uint32_t it = 0; it < my_items; ++it, item0 += gridDim.x) {
+    for (uint32_t s0 = 0; s0 < nslices; ++s0, ++k) {
+        // at most the operations issued during the previous PD-1 slices are outstanding: this wave's share of
+        // slice k (and of index words k+1) has landed; after the barrier everybody's has, and everybody is
+        // done with slice k-1, whose buffer slice k+PD goes into
+        if (k != 0) {
+            if (COUNT_STORES && stores_behind) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(COUNT_STORES ? (PD - 1) * DMA_OPS + EPI_STORES : 0) : "memory");
+            else asm volatile("s_waitcnt vmcnt(%0)" ::"n"((PD - 1) * DMA_OPS) : "memory");
+            stores_behind = false;
+            __syncthreads();
+        }
+        const bool fetch = k + PD < total;
+        const bool fetch_ix = k + PD + 1 < total;
+        const uint32_t lbp = buf >= 1 ? buf - 1 : NBUF - 1;
+        const uint32_t ibp = ibuf_next >= 1 ? ibuf_next - 1 : NIBUF - 1;
+        const uint32_t bbase = buf * SLICE + b_lane;
+
+        // Operand registers: the dense operand of a column group is re-armed with the next K-step's bytes as
+        // soon as its TM instructions have been issued; the sparse operand is double buffered.
+        v4i b_lo[TN], b_hi[TN];
+        v2i a_lo[2][TM], a_hi[2][TM];
+        uint32_t p_lo[2][TM], p_hi[2][TM];
+        auto issue_b = [&](auto ksc, auto cc) {
+            constexpr int ks = decltype(ksc)::value, c = decltype(cc)::value;
+            lds_read<((8 * ks) * WN + c * 16) * 16>(b_lo[c], bbase);
+            lds_read<((8 * ks + 4) * WN + c * 16) * 16>(b_hi[c], bbase);
+        };
+        auto issue_a = [&](auto ksc) {
+            constexpr int ks = decltype(ksc)::value;
+#pragma unroll
+            for (int t = 0; t < TM; ++t) {
+                const uint32_t e0 = __builtin_amdgcn_ubfe(iw_lo[t][ks], byte_shift, 8);
+                const uint32_t e1 = __builtin_amdgcn_ubfe(iw_hi[t][ks], byte_shift, 8);
+                lds_read64<0>(a_lo[ks & 1][t], e0);
+                lds_read32<8>(p_lo[ks & 1][t], e0);
+                lds_read64<0>(a_hi[ks & 1][t], e1);
+                lds_read32<12>(p_hi[ks & 1][t], e1);
+            }
+        };
+        // slice prologue: sparse operand first, then the dense operand of every column group, in this order
+        issue_a(std::integral_constant<int, 0>{});
+        static_for<0, TN>([&](auto cc) { issue_b(std::integral_constant<int, 0>{}, cc); });
+
+        static_for<0, KSTEPS>([&](auto ksc) {
+            constexpr int ks = decltype(ksc)::value;
+            constexpr bool LAST = ks + 1 == KSTEPS;
+            constexpr int RI = TM * IWORDS;  // index-word reads issued after column group 0 of the last K-step
+            static_for<0, TN>([&](auto cc) {
+                constexpr int c = decltype(cc)::value;
+                // LDS operations complete in order; the count is the number of operations issued after the
+                // ones this column group needs (see the issue order above and below)
+                if constexpr (c == 0) lgkm_wait<2 * (TN - 1)>();
+                else if constexpr (LAST) lgkm_wait<2 * (TN - 1 - c) + RI>();
+                else lgkm_wait<2 * TN + 4 * TM - 2>();
+                if constexpr (c == 0) {
+#pragma unroll
+                    for (int t = 0; t < TM; ++t)
+                        asm volatile("" : "+v"(a_lo[ks & 1][t]), "+v"(a_hi[ks & 1][t]), "+v"(p_lo[ks & 1][t]), "+v"(p_hi[ks & 1][t]));
+                }
+                asm volatile("" : "+v"(b_lo[c]), "+v"(b_hi[c]));
+                __builtin_amdgcn_sched_barrier(0);
+                const v8i bb = {b_lo[c][0], b_lo[c][1], b_lo[c][2], b_lo[c][3], b_hi[c][0], b_hi[c][1], b_hi[c][2], b_hi[c][3]};
+#pragma unroll
+                for (int t = 0; t < TM; ++t) {
+                    const v4i aa = {a_lo[ks & 1][t][0], a_lo[ks & 1][t][1], a_hi[ks & 1][t][0], a_hi[ks & 1][t][1]};
+                    acc[t][c] = __builtin_amdgcn_smfmac_i32_16x16x128_i8(aa, bb, acc[t][c], (int)(p_lo[ks & 1][t] | p_hi[ks & 1][t]), 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (!LAST) {
+                    issue_b(std::integral_constant<int, ks + 1>{}, cc);
+                    if constexpr (c == 0) issue_a(std::integral_constant<int, ks + 1>{});
+                } else if constexpr (c == 0) {
+                    read_ix(iw_raw, ibuf_next);  // the next slice's index words (this wave's own copy, landed)
+                }
+                // this slice's copy operations (slice k+PD of the table, index words k+PD+1), a few per column group
+                constexpr int IK = PD == 1 ? KSTEPS * TN / 2 : KSTEPS * TN;
+                constexpr int pos = ks * TN + c;
+                static_for<(pos < IK ? pos : IK) * DMA_OPS / IK, (pos + 1 < IK ? pos + 1 : IK) * DMA_OPS / IK>([&](auto oc) {
+                    constexpr int o = decltype(oc)::value;
+                    if constexpr (o < DMA_PER_WAVE) lut_op(lbp, fetch, std::integral_constant<int, o>{});
+                    else ix_op(ibp, fetch_ix, std::integral_constant<int, o - DMA_PER_WAVE>{});
+                });
+                __builtin_amdgcn_sched_barrier(0);
+            });
+        });
+        if (fetch) {
+            lut_advance();
+            if (fetch_ix) ix_advance();
+        }
+        unpack_ix(iw_lo, iw_hi, iw_raw);
+
+        buf = buf + 1 == NBUF ? 0 : buf + 1;
+        ibuf_next = ibuf_next + 1 == NIBUF ? 0 : ibuf_next + 1;
+    }
+    stores_behind = epilogue(item0);
+    }
+}
+
+template <int TN, int TM, int GS>
+int launch_sparse_tm(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_t* d_acc, uint32_t n,
+                     const Epilogue& ep)
+{
+    constexpr int LDS = sp_lds_bytes(TN, GS);
+    static_assert(2 * LDS <= 160 * 1024, "two workgroups per CU");
+    constexpr int TOK_ITEM = sp_tok_item(TM);
+    auto kern = gather_sparse_kernel<TN, TM, GS>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        int rc = hip_check(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, LDS),
+                           "hipFuncSetAttribute(gather_sparse)");
+        if (rc) return rc;
+        attr_set = true;
+    }
+    const uint32_t n_token_tiles = (n + TOK_ITEM - 1) / TOK_ITEM;
+    const uint32_t n_items = n_token_tiles * (a.g.M_pad / (16 * TN));
+    uint32_t grid = ctx->prop.multiProcessorCount * 2;
+    if (grid > n_items) grid = n_items;
+    const XcdMap xmap = choose_xcd_map(a.g.M_pad / (16 * TN), n_token_tiles, grid, (uint64_t)a.g.CB_pad * 16 * a.g.M_pad,
+                                       (uint64_t)n * a.g.idx_row_bytes);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(SP_THREADS), LDS, ctx->stream, d_idx, reinterpret_cast<const int8_t*>(a.d_lut),
+                       d_out, d_acc, n, a.g.M, a.g.CB_pad, a.g.idx_row_bytes, n_token_tiles, n_items, ep, xmap);
+    return hip_check(ctx, hipGetLastError(), "gather_sparse_kernel launch");
+}
+
+// 256-token items where the batch offers two of them per CU, else 128-token items (the rule of the dense kernel)
+template <int TN>
+int launch_sparse_tn(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_t* d_acc, uint32_t n, const Epilogue& ep)
+{
+    const uint64_t col_tiles = a.g.M_pad / (16 * TN);
+    const uint64_t items4 = (uint64_t)((n + sp_tok_item(4) - 1) / sp_tok_item(4)) * col_tiles;
+    const uint64_t items2 = (uint64_t)((n + sp_tok_item(2) - 1) / sp_tok_item(2)) * col_tiles;
+    const uint64_t slots = 2ull * ctx->prop.multiProcessorCount;
+    const bool small_items = items4 < slots || 10 * ((items2 + slots - 1) / slots) < 17 * ((items4 + slots - 1) / slots);
+    constexpr int GSB = TN <= 4 ? 32 : 16;  // 32-codebook slices in two buffers where two workgroups still fit a CU
+    if constexpr (GSB != 16) {
+        if (a.g.CB_pad % GSB == 0) {
+            if (small_items) return launch_sparse_tm<TN, 2, GSB>(ctx, a, d_idx, d_out, d_acc, n, ep);
+            return launch_sparse_tm<TN, 4, GSB>(ctx, a, d_idx, d_out, d_acc, n, ep);
+        }
+    }
+    if (small_items) return launch_sparse_tm<TN, 2, 16>(ctx, a, d_idx, d_out, d_acc, n, ep);
+    return launch_sparse_tm<TN, 4, 16>(ctx, a, d_idx, d_out, d_acc, n, ep);
+}
+
+}  // namespace
+
+uint32_t sparse_lds_bytes(uint32_t tn) { return (uint32_t)sp_lds_bytes((int)tn, 16); }
+
+int launch_gather_sparse(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_t* d_acc, uint32_t n,
+                         float scale, float lut_bias_term)
+{
+    Epilogue ep;
+    ep.scale = scale;
+    ep.lut_bias_term = lut_bias_term;
+    ep.bias = a.d_bias;
+    ep.act = a.desc.activation;
+    ep.op_scales = a.d_op_scales;
+    ep.op_col_tiles = a.op_col_tiles;
+    ep.op_idx_stride = a.op_idx_stride;
+    switch (a.g.q) {
+        case 3: return launch_sparse_tn<3>(ctx, a, d_idx, d_out, d_acc, n, ep);
+        case 4: return launch_sparse_tn<4>(ctx, a, d_idx, d_out, d_acc, n, ep);
+        case 6: return launch_sparse_tn<6>(ctx, a, d_idx, d_out, d_acc, n, ep);
+    }
+    return set_error(ctx, PIMDL_ERR_UNSUPPORTED, "no sparse gather kernel for %u column groups", a.g.q);
+}
+
+}  // namespace pimdl

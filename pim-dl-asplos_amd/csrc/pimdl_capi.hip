@@ -185,13 +185,17 @@ static void retile_lut_onehot(const int8_t* lut, int8_t* tiled, const AmmGeom& g
 {
     const uint32_t wn = g.col_block;
     const bool paired = g.C_tile == 8;
+    // position of column f % wn inside its tile: the sparse-instruction kernel deals a tile's columns to its
+    // 16-column groups so that a lane's accumulators are consecutive columns
+    std::vector<uint32_t> where(wn);
+    for (uint32_t s = 0; s < wn; ++s) where[g.gather_kind == 2 ? sparse_tile_column(wn / 16, s) : s] = s;
     for (uint32_t cb = 0; cb < g.CB; ++cb)
         for (uint32_t c = 0; c < g.C; ++c) {
             const int8_t* src = lut + ((size_t)cb * g.C + c) * g.M;
             const uint32_t entry = paired ? cb / 2 : cb, entries = paired ? g.CB_pad / 2 : g.CB_pad;
             const uint32_t slot = paired ? 8 * (cb & 1) + c : c;
             for (uint32_t f = 0; f < g.M; ++f)
-                tiled[((((size_t)(f / wn) * entries + entry) * wn) + f % wn) * 16 + slot] = src[f];
+                tiled[((((size_t)(f / wn) * entries + entry) * wn) + where[f % wn]) * 16 + slot] = src[f];
         }
 }
 
@@ -361,7 +365,7 @@ int pimdl_amm_create_tuned(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const flo
         delete a;
         return set_error(ctx, PIMDL_ERR_NOMEM, "pimdl_amm_create: host staging of %zu bytes failed", a->lut_bytes);
     }
-    if (i8 && g.gather_kind == 1) retile_lut_onehot(reinterpret_cast<const int8_t*>(lut), reinterpret_cast<int8_t*>(tiled.data()), g);
+    if (i8 && g.gather_kind != 0) retile_lut_onehot(reinterpret_cast<const int8_t*>(lut), reinterpret_cast<int8_t*>(tiled.data()), g);
     else if (i8) retile_lut(reinterpret_cast<const int8_t*>(lut), reinterpret_cast<int8_t*>(tiled.data()), g, row_elems);
     else if (grouped) {
         std::vector<float> wide;
@@ -457,13 +461,13 @@ int pimdl_amm_group_create(pimdl_ctx* ctx, pimdl_amm* const* amms, uint32_t coun
     if (!rc) rc = launch_ccs_prep(ctx, g, grp->d_centroids);
     if (!rc) rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, idx_buffer_bytes(g, max_n), "hipMalloc(index scratch)");
     // one gather launch for all members?
-    bool same = first->desc.lut_dtype == PIMDL_LUT_I8 && !first->grouped && first->g.gather_kind == 1 &&
+    bool same = first->desc.lut_dtype == PIMDL_LUT_I8 && !first->grouped && first->g.gather_kind != 0 &&
                 first->g.M % first->g.col_block == 0;
     const float lbt0 = first->desc.bias_mode == PIMDL_BIAS_TIMES_CB ? first->desc.lut_bias * (float)first->g.CB : first->desc.lut_bias;
     for (uint32_t i = 1; i < count && same; ++i) {
         const Amm* a = amms[i];
         const float lbt = a->desc.bias_mode == PIMDL_BIAS_TIMES_CB ? a->desc.lut_bias * (float)a->g.CB : a->desc.lut_bias;
-        same = a->desc.lut_dtype == PIMDL_LUT_I8 && !a->grouped && a->g.gather_kind == 1 && a->g.M == first->g.M &&
+        same = a->desc.lut_dtype == PIMDL_LUT_I8 && !a->grouped && a->g.gather_kind == first->g.gather_kind && a->g.M == first->g.M &&
                a->g.q == first->g.q && a->g.C_tile == first->g.C_tile && a->g.CB_pad == first->g.CB_pad &&
                a->lut_bytes == first->lut_bytes && a->desc.activation == first->desc.activation && lbt == lbt0;
     }

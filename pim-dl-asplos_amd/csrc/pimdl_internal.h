@@ -32,7 +32,9 @@ struct AmmGeom {
     uint32_t idx_tiled;     // layout of the packed index buffer, see above
     uint32_t lut_chunked;   // fp32 table of 32 centroids: [column block][codebook][8-byte chunk][row][2 floats]
     // gather kernel
-    uint32_t gather_kind;   // 0: byte-adder rows kernel, 1: one-hot matrix-core kernel (int8, C <= 16)
+    uint32_t gather_kind;   // 0: byte-adder rows kernel, 1: one-hot matrix-core kernel (int8, C <= 16),
+                            // 2: one-hot on the sparse matrix instruction (int8, 9 <= C <= 16; table laid out
+                            //    as for 1, with the columns of a tile permuted by sparse_tile_column)
     uint32_t q;             // 16-byte chunks per LUT row in LDS
     uint32_t col_block;     // columns per workgroup (int8: 16*q, fp32: 4*q)
     uint32_t row_pitch;     // bytes between LUT rows in LDS (16*q + 16: bank-conflict-free b128 gathers)
@@ -139,6 +141,13 @@ int launch_attention_hd64(Ctx* ctx, const float* d_q, const float* d_k, const fl
                           uint32_t seq, uint32_t heads, uint32_t in_stride, uint32_t out_stride, float scale);
 int launch_diag(Ctx* ctx, uint64_t bytes, float* copy_gbps, float* lds_gbps);
 int launch_diag_mfma_error(Ctx* ctx, uint32_t trials, float* max_err_u);
+
+// the sparse one-hot gather (gather_sp_kernel.hip)
+int launch_gather_sparse(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_t* d_acc_or_null,
+                         uint32_t n, float scale, float lut_bias_term);
+uint32_t sparse_tile_column(uint32_t tn, uint32_t s);  // column of a tile stored at position s of the tile
+uint32_t sparse_lds_bytes(uint32_t tn);
+bool gather_dense_only();
 
 uint32_t ccs_cb_per_wg(uint32_t v);  // codebooks one ccs workgroup covers (0: generic kernel)
 bool gather_rows_only();
