@@ -426,6 +426,7 @@ int launch_sparse_tm(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out,
     if (grid > n_items) grid = n_items;
     const XcdMap xmap = choose_xcd_map(a.g.M_pad / (16 * TN), n_token_tiles, grid, (uint64_t)a.g.CB_pad * 16 * a.g.M_pad,
                                        (uint64_t)n * a.g.idx_row_bytes);
+    snprintf(a.last_gather, sizeof(a.last_gather), "gather_sparse_kernel<%d, %d, %d>", TN, TM, GS);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(SP_THREADS), LDS, ctx->stream, d_idx, reinterpret_cast<const int8_t*>(a.d_lut),
                        d_out, d_acc, n, a.g.M, a.g.CB_pad, a.g.idx_row_bytes, n_token_tiles, n_items, ep, xmap);
     return hip_check(ctx, hipGetLastError(), "gather_sparse_kernel launch");

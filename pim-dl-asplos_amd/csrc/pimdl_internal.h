@@ -80,6 +80,8 @@ struct Amm {
     // several one-hot operators laid side by side along the columns (see Epilogue in gather_kernel.hip)
     float* d_op_scales;
     uint32_t op_col_tiles, op_idx_stride;
+    // name (with template arguments) of the gather kernel the operator's last launch used: what a profile lists
+    mutable char last_gather[80];
 };
 
 struct Ctx {
