@@ -128,6 +128,55 @@ PIMDL_API int pimdl_amm_create(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const
 PIMDL_API int pimdl_amm_create_tuned(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const float* centroids,
                                      const void* lut, const float* scales, const float* bias,
                                      uint32_t col_block, pimdl_amm** out);
+/* Every choice the library makes for an operator, open to a measured search (the tile autotuner).  The
+ * counterpart of the kernel_params the reference's auto-tuner enumerates -- sub-tile sizes, load tile sizes,
+ * LUT load type and loop order (inference-engine/src/tuner/auto_tuner.cpp:368-603) -- for this hardware:
+ * the token tile, the column block, the codebook group staged at a time, and the way entries are
+ * accumulated (which kernel).  0 in a field = the library's own choice.  Results do not depend on any of
+ * them (every kernel gives the same bits); only the time does. */
+typedef enum pimdl_gather_kernel {
+    PIMDL_GATHER_AUTO = 0,
+    PIMDL_GATHER_ROWS = 1,   /* byte adder: gathered row pieces summed by an identity matrix product; any C */
+    PIMDL_GATHER_ONEHOT = 2, /* one-hot x table on the dense int8 matrix instruction; C <= 16 */
+    PIMDL_GATHER_SPARSE = 3  /* one-hot as a 2:4 sparse operand, 8 codebooks per instruction; 9 <= C <= 16 */
+} pimdl_gather_kernel;
+typedef enum pimdl_search_kernel {
+    PIMDL_SEARCH_AUTO = 0,
+    PIMDL_SEARCH_SCAN = 1,      /* one lane per token, the reference's scan for every pair */
+    PIMDL_SEARCH_MFMA_F32 = 2,  /* scores on the fp32 matrix instruction, exact replay of near ties; C <= 16 */
+    PIMDL_SEARCH_MFMA_BF16 = 3  /* scores from three bf16 pieces per value; C <= 32, sub_vec_len 2, 4, 8 */
+} pimdl_search_kernel;
+typedef struct pimdl_amm_tuning {
+    uint32_t col_block;      /* output columns per work item of the gather: 48, 64 or 96 (what the kernel offers) */
+    uint32_t gather_kernel;  /* pimdl_gather_kernel; fixes the layout of the resident table */
+    uint32_t token_item;     /* tokens per work item of the matrix-core gathers: 128 or 256 */
+    uint32_t cb_per_slice;   /* codebooks staged in LDS at a time by the matrix-core gathers: 16 or 32
+                                (32 needs col_block <= 64 and num_codebook padded to a multiple of 32) */
+    uint32_t xcd_col_split;  /* how the 8 XCDs (each with its own L2) share the work items of the matrix-core
+                                gathers: 1, 2, 4 or 8 of them along the column tiles, the rest along the token
+                                tiles; PIMDL_XCD_PLAIN = no dealing.  A split that does not divide a launch's
+                                tile counts is replaced by the library's choice for that launch. */
+    uint32_t search_kernel;  /* pimdl_search_kernel */
+    uint32_t search_token_tile; /* tokens per tile of the bf16 matrix-core search: 64 or 128 */
+} pimdl_amm_tuning;
+#define PIMDL_XCD_PLAIN 0xFFFFFFFFu
+/* pimdl_amm_create with these choices made by the caller (tuning NULL or all zero: pimdl_amm_create).
+ * PIMDL_ERR_INVALID when the operator's shape has no kernel for a choice. */
+PIMDL_API int pimdl_amm_create_with(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const float* centroids,
+                                    const void* lut, const float* scales, const float* bias,
+                                    const pimdl_amm_tuning* tuning, pimdl_amm** out);
+/* Changes the choices that do not touch resident data (token_item, cb_per_slice, xcd_col_split,
+ * search_kernel, search_token_tile) on an existing operator, so that a search need not upload the table once per candidate;
+ * col_block and gather_kernel must be 0 or what the operator was created with.  pimdl_amm_get_tuning
+ * reports the operator's current settings (0 where the library still chooses per launch). */
+PIMDL_API int pimdl_amm_set_tuning(pimdl_amm* amm, const pimdl_amm_tuning* tuning);
+PIMDL_API int pimdl_amm_get_tuning(const pimdl_amm* amm, pimdl_amm_tuning* tuning);
+/* Replaces the operator's bias [M] (HOST pointer; NULL = zeros).  The reference's pim_lut reads
+ * bias_tensor anew on every call (src/host/pim_lut_host.cpp:201), so a caller may refill that buffer between
+ * calls; the C++ layer sends it through here each time.  Ordered behind the launches already queued on the
+ * context's stream; synchronous.  A fused group (pimdl_amm_group_run_fused) keeps the biases its members had
+ * when it was created. */
+PIMDL_API int pimdl_amm_set_bias(pimdl_amm* amm, const float* bias);
 PIMDL_API int pimdl_amm_destroy(pimdl_amm* amm);
 
 /* The AMM itself.  Replaces amm_host (src/host/amm_host.h:8-10, amm_host.cpp:10-30) =
@@ -204,7 +253,9 @@ PIMDL_API int pimdl_amm_index_calculation(pimdl_amm* amm, const float* in, uint3
                                           uint16_t* idx_out, uint32_t n_stile_size,
                                           uint32_t cb_mtile_size);
 /* pimdl_lut_gather replaces pim_lut (src/host/pim_lut_host.h:13-14, pim_lut_host.cpp:121-222):
- * idx is HOST uint16 row-major [n][CB] holding centroid ids; out is host or device fp32 [n][M]. */
+ * idx is HOST uint16 row-major [n][CB] holding centroid ids; out is host or device fp32 [n][M].
+ * PIMDL_ERR_INVALID (the text names token and codebook) when an entry is not below num_centroid, e.g. a
+ * buffer that pim_lut has already rewritten into table offsets (pim_lut_host.cpp:40-104). */
 PIMDL_API int pimdl_lut_gather(pimdl_amm* amm, const uint16_t* idx, uint32_t n, float* out);
 
 /* ---- the reference's DPU tile orders ---------------------------------------------------------

@@ -19,9 +19,11 @@
 // three are plain row-major / canonical.
 //
 // Differences from the reference, all deliberate:
-//   * the LUT is uploaded to the device once per (pointer, shape) and reused; the reference re-sends
-//     it on every call (pim_lut_host.cpp:143).  If the contents behind the same pointer change, call
-//     pimdl_host_invalidate(lut_table).  A sampled fingerprint catches most such changes anyway.
+//   * the LUT and the centroids are uploaded to the device once per (pointer, shape) and reused; the
+//     reference re-sends the LUT on every call (pim_lut_host.cpp:143).  Every call hashes both buffers
+//     in full (one pass over host memory) and uploads again when anything behind the pointers has
+//     changed; bias_tensor is sent on every call, as the reference reads it on every call (:201).
+//     pimdl_host_invalidate(lut_table) drops the device copy explicitly.
 //   * failures throw std::runtime_error (the reference aborts through DPU_ASSERT);
 //   * nothing is leaked per call (the reference leaks its index and int32 buffers,
 //     amm_host.cpp:19, pim_lut_host.cpp:133).

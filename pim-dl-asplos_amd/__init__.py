@@ -31,7 +31,8 @@ EXPORTS = ["pimdl_init", "pimdl_destroy", "pimdl_last_error", "pimdl_set_stream"
            "pimdl_amm_run_tiled", "pimdl_lut_gather_tiled", "pimdl_lutgen",
            "pimdl_layer_norm", "pimdl_get_device_info", "pimdl_amm_get_geometry", "pimdl_diag_bandwidth",
            "pimdl_diag_mfma_error", "pimdl_amm_group_create", "pimdl_amm_group_run", "pimdl_amm_group_destroy",
-           "pimdl_attention", "pimdl_amm_group_fused_cols", "pimdl_amm_group_run_fused", "pimdl_amm_run_noalloc"]
+           "pimdl_attention", "pimdl_amm_group_fused_cols", "pimdl_amm_group_run_fused", "pimdl_amm_run_noalloc", "pimdl_amm_set_bias",
+           "pimdl_amm_create_with", "pimdl_amm_set_tuning", "pimdl_amm_get_tuning"]
 NOALLOC_SCRATCH_BYTES = 8 << 20
 
 
@@ -62,6 +63,21 @@ class DeviceInfo(ctypes.Structure):
 class Tiling(ctypes.Structure):
     _fields_ = [(n, ctypes.c_uint32) for n in ("n_stile_size", "cb_mtile_size", "feature_stile_size",
                                                "feature_mtile_size")]
+
+
+TUNING_FIELDS = ("col_block", "gather_kernel", "token_item", "cb_per_slice", "xcd_col_split", "search_kernel",
+                 "search_token_tile")
+GATHER_AUTO, GATHER_ROWS, GATHER_ONEHOT, GATHER_SPARSE = 0, 1, 2, 3
+SEARCH_AUTO, SEARCH_SCAN, SEARCH_MFMA_F32, SEARCH_MFMA_BF16 = 0, 1, 2, 3
+XCD_PLAIN = 0xFFFFFFFF
+
+
+class AmmTuning(ctypes.Structure):
+    """pimdl_amm_tuning: the choices a measured search may take over from the library (0 = library's choice)."""
+    _fields_ = [(n, ctypes.c_uint32) for n in TUNING_FIELDS]
+
+    def asdict(self):
+        return {n: int(getattr(self, n)) for n in TUNING_FIELDS}
 
 
 class AmmGeometry(ctypes.Structure):
@@ -259,10 +275,12 @@ class Context:
         return AmmGroup(self, amms)
 
     def amm(self, centroids, lut, scales=None, bias=None, max_n=8192, lut_bias=0.0, bias_mode=BIAS_ONCE,
-            scale_group=0, col_block=0, activation=ACT_NONE):
+            scale_group=0, col_block=0, activation=ACT_NONE, tuning=None):
         """col_block: width of the gather kernel's column tile (0 = chosen by the library).
-        activation: ACT_GELU_TANH applies the tanh form of GELU to the output inside the gather's epilogue."""
-        return Amm(self, centroids, lut, scales, bias, max_n, lut_bias, bias_mode, scale_group, col_block, activation)
+        activation: ACT_GELU_TANH applies the tanh form of GELU to the output inside the gather's epilogue.
+        tuning: dict over TUNING_FIELDS (pimdl_amm_tuning), the choices a measured search takes over."""
+        return Amm(self, centroids, lut, scales, bias, max_n, lut_bias, bias_mode, scale_group, col_block, activation,
+                   tuning)
 
 
 class AmmGroup:
@@ -311,7 +329,7 @@ class Amm:
     """One LUT-AMM operator resident in HBM."""
 
     def __init__(self, ctx, centroids, lut, scales, bias, max_n, lut_bias, bias_mode, scale_group, col_block=0,
-                 activation=0):
+                 activation=0, tuning=None):
         centroids = np.ascontiguousarray(centroids, np.float32)
         CB, C, v = centroids.shape
         lut = np.ascontiguousarray(lut)
@@ -328,8 +346,22 @@ class Amm:
             bias = np.ascontiguousarray(bias, np.float32)
             assert bias.shape == (M,)
         self._h = ctypes.c_void_p()
-        ctx._check(lib().pimdl_amm_create_tuned(ctx._h, ctypes.byref(desc), _ptr(centroids), _ptr(lut), _ptr(scales),
-                                                _ptr(bias), col_block, ctypes.byref(self._h)))
+        tune = AmmTuning(**dict(tuning or {}))
+        if col_block:
+            tune.col_block = col_block
+        ctx._check(lib().pimdl_amm_create_with(ctx._h, ctypes.byref(desc), _ptr(centroids), _ptr(lut), _ptr(scales),
+                                               _ptr(bias), ctypes.byref(tune), ctypes.byref(self._h)))
+
+    def set_tuning(self, **fields):
+        """The choices that do not touch resident data: token_item, cb_per_slice, xcd_col_split, search_kernel,
+        search_token_tile (fields left out go back to the library's choice)."""
+        tune = AmmTuning(**fields)
+        self.ctx._check(lib().pimdl_amm_set_tuning(self._h, ctypes.byref(tune)))
+
+    def tuning(self):
+        tune = AmmTuning()
+        self.ctx._check(lib().pimdl_amm_get_tuning(self._h, ctypes.byref(tune)))
+        return tune.asdict()
 
     def close(self):
         if self._h and self.ctx._h:
@@ -409,6 +441,13 @@ class Amm:
         til = Tiling(n_stile, cb_mtile, f_stile, f_mtile)
         self.ctx._check(lib().pimdl_lut_gather_tiled(self._h, _ptr(idx_flat), n, _ptr(out), ctypes.byref(til)))
         return out
+
+    def set_bias(self, bias):
+        """Replace the operator's bias [M] (None: zeros)."""
+        if bias is not None:
+            bias = np.ascontiguousarray(bias, np.float32)
+            assert bias.shape == (self.M,)
+        self.ctx._check(lib().pimdl_amm_set_bias(self._h, _ptr(bias)))
 
     def lut_gather(self, idx):
         idx = np.ascontiguousarray(idx, np.uint16)

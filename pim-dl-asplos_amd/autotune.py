@@ -1,32 +1,57 @@
 """Measured tile search for a LUT-AMM operator.
 
-The reference ships an auto-tuner that enumerates DPU tilings and ranks them with an analytic latency
-model of UPMEM hardware (inference-engine/src/tuner/auto_tuner.cpp:368-603; input and output are YAML files,
-:793-820).  That model has no meaning on a GPU, so the counterpart here measures: for one operator shape it
-builds the operator with every column-tile width the gather kernel offers, times the two kernels with
-events on the device (pimdl_amm_profile) and keeps the fastest.  The result is cached in a JSON file keyed
-by device and shape, and can be written in the reference's single-kernel YAML layout with the chosen tile
-under kernel_params.
+The reference ships an auto-tuner that enumerates DPU tilings x micro-kernel parameters (sub-tile sizes, load
+tile sizes, LUT load type, loop order) and ranks them with an analytic latency model of UPMEM hardware
+(inference-engine/src/tuner/auto_tuner.cpp:368-603; input and output are YAML files, :793-820).  That model has
+no meaning on a GPU, so the counterpart here measures.  For one operator shape it enumerates what the library
+would otherwise decide by rule (pimdl_amm_tuning):
+
+    gather_kernel   how entries are accumulated: byte adder / dense one-hot / sparse one-hot matrix kernel
+    col_block       output columns per work item (48, 64, 96)
+    token_item      tokens per work item (128, 256)
+    cb_per_slice    codebooks staged in LDS at a time (16, 32)
+    xcd_col_split   how the 8 XCDs share column tiles and token tiles (1, 2, 4, 8, plain order)
+    search_kernel   closest-centroid search: lane-per-token scan / fp32 matrix core / bf16 matrix core
+    search_token_tile  tokens per tile of the bf16 search (64, 128)
+
+times the two kernels with events on the device (pimdl_amm_profile) and keeps the fastest setting of each
+kernel.  Gather and search are independent (they only share the packed index layout, which depends on the
+gather kernel), so the search space is a sum, not a product: every (gather_kernel, col_block) pair costs one
+table upload, the other gather knobs and all search knobs are switched on the resident operator.  Every
+candidate gives the same output bits; `tune` checks that on the way.  The result is cached in a JSON file keyed
+by device and shape, and can be written in the reference's single-kernel YAML layout with the choice under
+kernel_params.
 
     python autotune.py --n 8192 --k 768 --m 3072 --vec_len 4 --ncentroids 16 [--cache tiles.json] [--yaml out.yaml]
 """
 import argparse
+import itertools
 import json
 import os
 import sys
 
 import numpy as np
 
-CANDIDATES = (0, 48, 64, 96)   # 0 = the library's own load-balance choice
+COL_BLOCKS = (48, 64, 96)
+GATHER_KERNELS = {"rows": 1, "onehot": 2, "sparse": 3}
+SEARCH_KERNELS = {"scan": 1, "mfma_f32": 2, "mfma_bf16": 3}
+XCD_PLAIN = 0xFFFFFFFF
+RUNTIME_GATHER = {"token_item": (128, 256), "cb_per_slice": (16, 32), "xcd_col_split": (1, 2, 4, 8, XCD_PLAIN)}
 
 
 def shape_key(device, n, K, v, C, M, dtype):
     return f"{device}|n={n}|k={K}|v={v}|c={C}|m={M}|{dtype}"
 
 
-def tune(ctx, pimdl, n, K, v, C, M, lut_dtype="int8", seed=0, iters=20, candidates=CANDIDATES):
-    """Returns (best col_block, {col_block: {"ccs_ms", "gather_ms", "total_ms"}}); widths the operator's
-    kernel does not offer are skipped."""
+def _label(setting):
+    return ",".join(f"{k}={'plain' if v == XCD_PLAIN else v}" for k, v in sorted(setting.items())) or "library"
+
+
+def tune(ctx, pimdl, n, K, v, C, M, lut_dtype="int8", seed=0, iters=20, full=True):
+    """Returns (best, results).
+    best: {"gather": {tuning fields}, "search": {tuning fields}, "gather_ms", "ccs_ms", "library_gather_ms",
+    "library_ccs_ms"}; results: {label: {"gather_ms" or "ccs_ms", ...}} for every candidate that the operator's
+    shape has a kernel for.  full=False restricts the search to the column tile (one upload per width)."""
     import torch
     rng = np.random.default_rng(seed)
     CB = K // v
@@ -39,29 +64,94 @@ def tune(ctx, pimdl, n, K, v, C, M, lut_dtype="int8", seed=0, iters=20, candidat
         scales = None
     x = torch.randn((n, K), device="cuda", dtype=torch.float32)
     y = torch.empty((n, M), device="cuda", dtype=torch.float32)
-    results = {}
-    for cb in candidates:
+
+    def timed(amm):
+        t = amm.profile(x.data_ptr(), n, y.data_ptr(), warmup=3, iters=iters)
+        return t["ccs_ms"], t["gather_ms"]
+
+    def build(**fields):
         try:
-            amm = ctx.amm(cent, lut, scales, None, max_n=n, col_block=cb)
+            return ctx.amm(cent, lut, scales, None, max_n=n, tuning=fields)
         except pimdl.PimdlError as e:
             if e.code == pimdl.ERR_INVALID:
-                continue  # no kernel variant of that width for this operator
+                return None  # no kernel for that choice at this shape
             raise
-        t = amm.profile(x.data_ptr(), n, y.data_ptr(), warmup=3, iters=iters)
-        geo = amm.geometry()
-        results[cb] = {"ccs_ms": t["ccs_ms"], "gather_ms": t["gather_ms"], "total_ms": t["total_ms"],
-                       "col_block": geo["col_block"]}
+
+    results = {}
+    # the library's own choice: the baseline every candidate is compared with, and the reference output
+    amm = build()
+    lib_ccs, lib_gather = timed(amm)
+    lib_tuning = amm.tuning()
+    ref_out = y.clone()
+    results["library"] = {"ccs_ms": lib_ccs, "gather_ms": lib_gather, "tuning": lib_tuning}
+    # ---- search kernel (on the library's operator: the index layout does not depend on it) ----
+    best_search, best_ccs = {}, lib_ccs
+    for name, sk in (SEARCH_KERNELS.items() if full else ()):
+        for tile in ((0,) if sk != 3 else (64, 128)):
+            setting = {"search_kernel": sk, **({"search_token_tile": tile} if tile else {})}
+            try:
+                amm.set_tuning(**setting)
+            except pimdl.PimdlError as e:
+                if e.code == pimdl.ERR_INVALID:
+                    continue
+                raise
+            ccs_ms, _ = timed(amm)
+            assert torch.equal(y, ref_out), f"search setting {setting} changed the output"
+            results["search:" + _label(setting)] = {"ccs_ms": ccs_ms}
+            if ccs_ms < best_ccs:
+                best_search, best_ccs = setting, ccs_ms
+    amm.close()
+    # ---- gather: one upload per (kernel, column tile), run-time knobs on the resident operator ----
+    best_gather, best_gather_ms = {}, lib_gather
+    kernels = GATHER_KERNELS.items() if full else [("library", 0)]
+    for (kname, gk), cb in itertools.product(kernels, COL_BLOCKS):
+        base = {"col_block": cb, **({"gather_kernel": gk} if gk else {})}
+        amm = build(**base)
+        if amm is None:
+            continue
+        runtime = [{}]
+        if full:
+            runtime += [{k: val} for k, vals in RUNTIME_GATHER.items() for val in vals]
+        best_rt = {}
+        for rt in runtime:
+            try:
+                amm.set_tuning(**rt)
+            except pimdl.PimdlError as e:
+                if e.code == pimdl.ERR_INVALID:
+                    continue
+                raise
+            _, g_ms = timed(amm)
+            assert torch.equal(y, ref_out), f"gather setting {base} {rt} changed the output"
+            results["gather:" + _label({**base, **rt})] = {"gather_ms": g_ms}
+            if g_ms < best_gather_ms:
+                best_gather, best_gather_ms, best_rt = {**base, **rt}, g_ms, rt
+        # the run-time knobs are searched one at a time; try the best of each together
+        if full and len(runtime) > 1:
+            combo = {}
+            for k in RUNTIME_GATHER:
+                cands = [(results["gather:" + _label({**base, k: val})]["gather_ms"], val) for val in RUNTIME_GATHER[k]
+                         if "gather:" + _label({**base, k: val}) in results]
+                if cands and min(cands)[0] < results["gather:" + _label(base)]["gather_ms"]:
+                    combo[k] = min(cands)[1]
+            if len(combo) > 1:
+                try:
+                    amm.set_tuning(**combo)
+                    _, g_ms = timed(amm)
+                    assert torch.equal(y, ref_out)
+                    results["gather:" + _label({**base, **combo})] = {"gather_ms": g_ms}
+                    if g_ms < best_gather_ms:
+                        best_gather, best_gather_ms = {**base, **combo}, g_ms
+                except pimdl.PimdlError as e:
+                    if e.code != pimdl.ERR_INVALID:
+                        raise
         amm.close()
-    if not results:
-        raise RuntimeError("no candidate could be built")
-    # the fastest explicit width; "auto" (0) only documents what the library would have picked
-    explicit = [c for c in results if c != 0]
-    best = min(explicit, key=lambda c: results[c]["gather_ms"]) if explicit else results[0]["col_block"]
+    best = {"gather": best_gather, "search": best_search, "gather_ms": best_gather_ms, "ccs_ms": best_ccs,
+            "library_gather_ms": lib_gather, "library_ccs_ms": lib_ccs}
     return best, results
 
 
 class TileCache:
-    """JSON file {shape key: col_block}."""
+    """JSON file {shape key: tuning fields}."""
 
     def __init__(self, path):
         self.path = path
@@ -71,23 +161,24 @@ class TileCache:
                 self.table = json.load(f)
 
     def get(self, key):
-        return int(self.table.get(key, 0))
+        """Tuning fields to pass as Context.amm(..., tuning=...); {} when the shape was never tuned."""
+        return dict(self.table.get(key, {}))
 
-    def put(self, key, col_block):
-        self.table[key] = int(col_block)
+    def put(self, key, best):
+        self.table[key] = {**best["gather"], **best["search"]}
         if self.path:
             with open(self.path, "w") as f:
                 json.dump(self.table, f, indent=1, sort_keys=True)
 
 
-def write_yaml(path, n, K, v, C, M, col_block, timing):
+def write_yaml(path, n, K, v, C, M, best):
     """The reference's single-kernel YAML layout (inference-engine/configs/single_kernel_output_example.yaml)
-    with the measured choice; the DPU-only keys are left out."""
+    with the measured choice under kernel_params; the DPU-only keys are left out."""
     import yaml
     doc = {"amm_shape_params": {"n": n, "input_feature_len": K, "num_codebook": K // v, "num_centroid": C,
                                 "output_feature_len": M, "scale": 0.1, "bias": 0.0},
-           "kernel_params": {"col_block": int(col_block), "gather_ms": float(timing["gather_ms"]),
-                             "ccs_ms": float(timing["ccs_ms"])}}
+           "kernel_params": {**{k: int(val) for k, val in {**best["gather"], **best["search"]}.items()},
+                             "gather_ms": float(best["gather_ms"]), "ccs_ms": float(best["ccs_ms"])}}
     with open(path, "w") as f:
         yaml.safe_dump(doc, f, sort_keys=False)
 
@@ -100,6 +191,8 @@ def main(argv=None):
     ap.add_argument("--vec_len", type=int, default=4)
     ap.add_argument("--ncentroids", type=int, default=16)
     ap.add_argument("--lut_dtype", choices=("int8", "fp32"), default="int8")
+    ap.add_argument("--iters", type=int, default=20)
+    ap.add_argument("--col_block_only", action="store_true", help="search the column tile only")
     ap.add_argument("--cache", type=str, default=None)
     ap.add_argument("--yaml", type=str, default=None)
     args = ap.parse_args(argv)
@@ -109,19 +202,23 @@ def main(argv=None):
     pimdl = load_package()
     ctx = pimdl.Context(0)
     try:
-        best, results = tune(ctx, pimdl, args.n, args.k, args.vec_len, args.ncentroids, args.m, args.lut_dtype)
+        best, results = tune(ctx, pimdl, args.n, args.k, args.vec_len, args.ncentroids, args.m, args.lut_dtype,
+                             iters=args.iters, full=not args.col_block_only)
         dev = ctx.device_info()["name"]
     finally:
         ctx.close()
-    for cb, r in sorted(results.items()):
-        print(f"col_block {cb if cb else 'auto(' + str(r['col_block']) + ')':>9}: search {r['ccs_ms'] * 1e3:7.1f} us, "
-              f"gather {r['gather_ms'] * 1e3:7.1f} us")
-    print(f"best col_block: {best}")
+    for label, r in results.items():
+        which = "gather_ms" if label.startswith("gather") else "ccs_ms" if label.startswith("search") else None
+        if which:
+            print(f"{label:<72} {r[which] * 1e3:8.1f} us")
+        else:
+            print(f"{label:<72} search {r['ccs_ms'] * 1e3:.1f} us, gather {r['gather_ms'] * 1e3:.1f} us  {r['tuning']}")
+    print(f"best gather: {_label(best['gather'])}  {best['gather_ms'] * 1e3:.1f} us (library {best['library_gather_ms'] * 1e3:.1f} us)")
+    print(f"best search: {_label(best['search'])}  {best['ccs_ms'] * 1e3:.1f} us (library {best['library_ccs_ms'] * 1e3:.1f} us)")
     if args.cache:
         TileCache(args.cache).put(shape_key(dev, args.n, args.k, args.vec_len, args.ncentroids, args.m, args.lut_dtype), best)
     if args.yaml:
-        write_yaml(args.yaml, args.n, args.k, args.vec_len, args.ncentroids, args.m, best,
-                   results[best] if best in results else results[0])
+        write_yaml(args.yaml, args.n, args.k, args.vec_len, args.ncentroids, args.m, best)
     return 0
 
 

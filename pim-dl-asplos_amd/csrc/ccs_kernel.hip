@@ -1114,7 +1114,7 @@ int launch_ccs_t(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_ce
     const int vec_ok = (g.K % 4 == 0) && ((reinterpret_cast<uintptr_t>(d_x) & 15) == 0);
     const float* aux = d_cent + (size_t)g.CB * g.C * g.v;
     const float* cnmax = aux + ccs_aux_floats(g);
-    if (ccs_exact_only())
+    if (g.tune_search ? g.tune_search == PIMDL_SEARCH_SCAN : ccs_exact_only())
         hipLaunchKernelGGL((ccs_kernel<V, IDX_BITS, false>), grid, dim3(CCS_THREADS), 0, ctx->stream, d_x, d_cent,
                            aux, cnmax, d_idx, n, g.K, g.CB, g.C, g.idx_row_bytes, (int)g.idx_tiled, vec_ok, g.CB_pad, tiles_cb, total);
     else
@@ -1205,7 +1205,8 @@ int launch_ccs_bf16(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d
     const uint64_t tiles128 = (uint64_t)((n + 127) / 128) * (g.CB_pad / CcsMfmaShape<V, WIDE>::RCB);
     // (measured: 7.4 -> 5.9 us at 192 tiles, 8.7 -> 6.9 us at 384, equal at 768 = one per resident workgroup,
     // 10 % slower beyond)
-    if (tiles128 < 3ull * ctx->prop.multiProcessorCount) return launch_ccs_bf16_tt<V, WIDE, 64>(ctx, g, d_x, d_cent, d_idx, n, x_cols);
+    const bool small_tiles = g.tune_search_tile ? g.tune_search_tile == 64 : tiles128 < 3ull * ctx->prop.multiProcessorCount;
+    if (small_tiles) return launch_ccs_bf16_tt<V, WIDE, 64>(ctx, g, d_x, d_cent, d_idx, n, x_cols);
     return launch_ccs_bf16_tt<V, WIDE, 128>(ctx, g, d_x, d_cent, d_idx, n, x_cols);
 }
 
@@ -1213,7 +1214,10 @@ template <int IDX_BITS>
 int launch_ccs_bits(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_cent, uint8_t* d_idx, uint32_t n,
                     uint32_t x_cols)
 {
-    if (IDX_BITS == 8 && g.C <= 32 && !ccs_exact_only() && !ccs_f32_only()) {
+    // the operator's own choice (pimdl_amm_tuning.search_kernel) comes before the environment's
+    const bool exact = g.tune_search ? g.tune_search == PIMDL_SEARCH_SCAN : ccs_exact_only();
+    const bool f32 = g.tune_search ? g.tune_search == PIMDL_SEARCH_MFMA_F32 : ccs_f32_only();
+    if (IDX_BITS == 8 && g.C <= 32 && !exact && !f32) {
         switch (g.v) {
             case 2: return launch_ccs_bf16<2, true>(ctx, g, d_x, d_cent, d_idx, n, x_cols);
             case 4: return launch_ccs_bf16<4, true>(ctx, g, d_x, d_cent, d_idx, n, x_cols);
@@ -1221,8 +1225,8 @@ int launch_ccs_bits(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d
             default: break;
         }
     }
-    if (IDX_BITS == 4 && !ccs_exact_only()) {
-        if (!ccs_f32_only()) {
+    if (IDX_BITS == 4 && !exact) {
+        if (!f32) {
             switch (g.v) {
                 case 2: return launch_ccs_bf16<2, false>(ctx, g, d_x, d_cent, d_idx, n, x_cols);
                 case 4: return launch_ccs_bf16<4, false>(ctx, g, d_x, d_cent, d_idx, n, x_cols);
@@ -1232,7 +1236,7 @@ int launch_ccs_bits(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d
         }
     }
     if (x_cols) return set_error(ctx, PIMDL_ERR_UNSUPPORTED, "shared-input search needs the matrix-core search kernel");
-    if (IDX_BITS == 4 && !ccs_exact_only()) {
+    if (IDX_BITS == 4 && !exact) {
         switch (g.v) {
             case 2: return launch_ccs_mfma<2>(ctx, g, d_x, d_cent, d_idx, n);
             case 4: return launch_ccs_mfma<4>(ctx, g, d_x, d_cent, d_idx, n);
@@ -1426,7 +1430,8 @@ int launch_ccs(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d_cent
 // matrix-core kernel and whole codebook tiles per operator.
 bool ccs_supports_shared_input(const AmmGeom& g, uint32_t x_cols)
 {
-    if (!ccs_has_bf16(g) || ccs_exact_only() || ccs_f32_only()) return false;
+    if (!ccs_has_bf16(g)) return false;
+    if (g.tune_search ? g.tune_search != PIMDL_SEARCH_MFMA_BF16 : (ccs_exact_only() || ccs_f32_only())) return false;
     const uint32_t tf = (ccs_bf16_wide(g) ? 8 : 16) * g.v;
     return x_cols % tf == 0;
 }

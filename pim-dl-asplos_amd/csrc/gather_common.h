@@ -47,11 +47,14 @@ struct XcdMap {
 };
 
 // Picks the split with the least L2 fill traffic: 8 * (lut_bytes / col_split + idx_bytes / tok_split).
+// forced: the caller's column split (pimdl_amm_tuning.xcd_col_split), used when it divides the tile counts
 inline XcdMap choose_xcd_map(uint32_t n_col_tiles, uint32_t n_token_tiles, uint32_t grid, uint64_t lut_bytes,
-                             uint64_t idx_bytes)
+                             uint64_t idx_bytes, uint32_t forced = 0)
 {
     XcdMap best{0, 0, 0};
-    if (grid % 8 != 0) return best;
+    if (grid % 8 != 0 || forced == PIMDL_XCD_PLAIN) return best;
+    if (forced && n_col_tiles % forced == 0 && n_token_tiles % (8 / forced) == 0)
+        return XcdMap{forced, 8 / forced, n_token_tiles / (8 / forced)};
     uint64_t best_cost = lut_bytes + idx_bytes / 8 + 1;  // plain order: every XCD reads the whole LUT
     best_cost *= 8;
     for (uint32_t cs = 8; cs >= 1; cs /= 2) {

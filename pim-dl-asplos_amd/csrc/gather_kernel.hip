@@ -807,7 +807,8 @@ int launch_onehot_tm(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out,
     if (grid > n_items) grid = n_items;
     const uint32_t slice_entries = P8 ? a.g.CB_pad / 2 : a.g.CB_pad;  // codebooks, or pairs of them
     const XcdMap xmap = choose_xcd_map(a.g.M_pad / (16 * TN), n_token_tiles, grid,
-                                       (uint64_t)slice_entries * 16 * a.g.M_pad, (uint64_t)n * a.g.idx_row_bytes);
+                                       (uint64_t)slice_entries * 16 * a.g.M_pad, (uint64_t)n * a.g.idx_row_bytes,
+                                       a.g.tune_xcd_col_split);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(OH_THREADS), LDS, ctx->stream, d_idx,
                        reinterpret_cast<const int8_t*>(a.d_lut), d_out, d_acc, n, a.g.M, slice_entries,
                        a.g.idx_row_bytes, n_token_tiles, n_items, ep, xmap);
@@ -829,10 +830,11 @@ int launch_onehot(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, in
     constexpr int GSB = (TN == 3 || (TN == 4 && !P8)) ? 32 : 16;
     const uint64_t slots = 2ull * ctx->prop.multiProcessorCount;
     const uint64_t items2 = (uint64_t)((n + oh_tok_item(2) - 1) / oh_tok_item(2)) * (a.g.M_pad / (16 * TN));
-    const bool small_items = items4 < slots || 10 * ((items2 + slots - 1) / slots) < 17 * ((items4 + slots - 1) / slots);
+    bool small_items = items4 < slots || 10 * ((items2 + slots - 1) / slots) < 17 * ((items4 + slots - 1) / slots);
+    if (a.g.tune_token_item) small_items = a.g.tune_token_item == 128;
     if constexpr (GSB != 16) {
         const uint32_t entries = P8 ? a.g.CB_pad / 2 : a.g.CB_pad;
-        if (entries % GSB == 0) {
+        if (entries % GSB == 0 && a.g.tune_cb_per_slice != 16) {
             if (small_items) return launch_onehot_tm<TN, 2, P8, GSB>(ctx, a, d_idx, d_out, d_acc, n, ep);
             return launch_onehot_tm<TN, 4, P8, GSB>(ctx, a, d_idx, d_out, d_acc, n, ep);
         }
@@ -1166,8 +1168,53 @@ bool gather_dense_only()
     return v;
 }
 
-bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::string* why, uint32_t col_block_hint)
+bool apply_runtime_tuning(AmmGeom* g, const pimdl_amm_tuning& t, std::string* why)
 {
+    const bool matrix_core = g->gather_kind != 0;
+    if (t.token_item && (!matrix_core || (t.token_item != 128 && t.token_item != 256))) {
+        *why = "token_item must be 128 or 256, and only the matrix-core gathers (int8, up to 16 centroids) have it";
+        return false;
+    }
+    if (t.cb_per_slice) {
+        const uint32_t entries = g->C_tile == 8 ? g->CB_pad / 2 : g->CB_pad;  // codebooks, or pairs of them
+        const bool has32 = g->gather_kind == 2 ? g->q <= 4 : (g->q == 3 || (g->q == 4 && g->C_tile != 8));
+        if (!matrix_core || (t.cb_per_slice != 16 && !(t.cb_per_slice == 32 && has32 && entries % 32 == 0))) {
+            *why = "cb_per_slice must be 16, or 32 where the operator's kernel has that variant";
+            return false;
+        }
+    }
+    if (t.xcd_col_split && t.xcd_col_split != PIMDL_XCD_PLAIN &&
+        (!matrix_core || (t.xcd_col_split != 1 && t.xcd_col_split != 2 && t.xcd_col_split != 4 && t.xcd_col_split != 8))) {
+        *why = "xcd_col_split must be 1, 2, 4, 8 or PIMDL_XCD_PLAIN, and only the matrix-core gathers have it";
+        return false;
+    }
+    if (t.search_kernel > PIMDL_SEARCH_MFMA_BF16) { *why = "unknown search_kernel"; return false; }
+    const bool v248 = g->v == 2 || g->v == 4 || g->v == 8;
+    if (t.search_kernel == PIMDL_SEARCH_MFMA_F32 && !(g->C <= 16 && v248)) {
+        *why = "the fp32 matrix-core search needs up to 16 centroids and sub_vec_len 2, 4 or 8";
+        return false;
+    }
+    if (t.search_kernel == PIMDL_SEARCH_MFMA_BF16 && !(g->C <= 32 && v248)) {
+        *why = "the bf16 matrix-core search needs up to 32 centroids and sub_vec_len 2, 4 or 8";
+        return false;
+    }
+    if (t.search_token_tile && t.search_token_tile != 64 && t.search_token_tile != 128) {
+        *why = "search_token_tile must be 64 or 128";
+        return false;
+    }
+    g->tune_search_tile = t.search_token_tile;
+    g->tune_token_item = t.token_item;
+    g->tune_cb_per_slice = t.cb_per_slice;
+    g->tune_xcd_col_split = t.xcd_col_split;
+    g->tune_search = t.search_kernel;
+    return true;
+}
+
+bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::string* why, const pimdl_amm_tuning* tuning)
+{
+    const pimdl_amm_tuning none = {0, 0, 0, 0, 0, 0, 0};
+    const pimdl_amm_tuning& tune = tuning ? *tuning : none;
+    const uint32_t col_block_hint = tune.col_block;
     const uint32_t K = d.input_feature_len, v = d.sub_vec_len, C = d.num_centroid, M = d.output_feature_len;
     if (!K || !v || !C || !M || !d.max_n) { *why = "zero-sized dimension"; return false; }
     if (K % v) { *why = "input_feature_len is not a multiple of sub_vec_len"; return false; }
@@ -1186,6 +1233,21 @@ bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::s
     g->q = ct >= 128 ? 2 : 4;
     g->gather_kind = (i8 && C <= 16 && !gather_rows_only()) ? 1 : 0;
     if (g->gather_kind == 1 && C > 8 && !gather_dense_only()) g->gather_kind = 2;
+    switch (tune.gather_kernel) {
+        case PIMDL_GATHER_AUTO: break;
+        case PIMDL_GATHER_ROWS:
+            g->gather_kind = 0;
+            break;
+        case PIMDL_GATHER_ONEHOT:
+            if (!(i8 && C <= 16)) { *why = "the one-hot gather needs an int8 table with up to 16 centroids"; return false; }
+            g->gather_kind = 1;
+            break;
+        case PIMDL_GATHER_SPARSE:
+            if (!(i8 && C > 8 && C <= 16)) { *why = "the sparse one-hot gather needs an int8 table with 9 to 16 centroids"; return false; }
+            g->gather_kind = 2;
+            break;
+        default: *why = "unknown gather_kernel"; return false;
+    }
     g->idx_tiled = g->gather_kind != 0;
     if (g->gather_kind != 0) {
         // One-hot matrix-core kernel: an item is 256 tokens x 16*TN columns, all items cost the
@@ -1226,7 +1288,7 @@ bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::s
         g->ccs_cb_per_wg = ccs_cb_per_wg(v);
         g->ccs_row_floats = g->ccs_cb_per_wg * v;
         g->ccs_lds_bytes = g->ccs_cb_per_wg ? 64 * (g->ccs_row_floats + 4) * 4 : 0;
-        return true;
+        return apply_runtime_tuning(g, tune, why);
     }
     if (i8 && ct >= 16 && ct <= 64) {
         // Column block of 64 or 48 columns: take the one that fills the persistent grid (two
@@ -1271,7 +1333,8 @@ bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::s
     g->ccs_cb_per_wg = ccs_cb_per_wg(v);
     g->ccs_row_floats = g->ccs_cb_per_wg * v;
     g->ccs_lds_bytes = g->ccs_cb_per_wg ? 64 * (g->ccs_row_floats + 4) * 4 : 0;
-    return true;
+    if (col_block_hint && !i8) { *why = "fp32 tables have one column block width"; return false; }
+    return apply_runtime_tuning(g, tune, why);
 }
 
 int launch_gather(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_t* d_acc, uint32_t n)

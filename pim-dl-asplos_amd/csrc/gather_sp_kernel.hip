@@ -425,7 +425,7 @@ int launch_sparse_tm(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out,
     uint32_t grid = ctx->prop.multiProcessorCount * 2;
     if (grid > n_items) grid = n_items;
     const XcdMap xmap = choose_xcd_map(a.g.M_pad / (16 * TN), n_token_tiles, grid, (uint64_t)a.g.CB_pad * 16 * a.g.M_pad,
-                                       (uint64_t)n * a.g.idx_row_bytes);
+                                       (uint64_t)n * a.g.idx_row_bytes, a.g.tune_xcd_col_split);
     snprintf(a.last_gather, sizeof(a.last_gather), "gather_sparse_kernel<%d, %d, %d>", TN, TM, GS);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(SP_THREADS), LDS, ctx->stream, d_idx, reinterpret_cast<const int8_t*>(a.d_lut),
                        d_out, d_acc, n, a.g.M, a.g.CB_pad, a.g.idx_row_bytes, n_token_tiles, n_items, ep, xmap);
@@ -440,10 +440,11 @@ int launch_sparse_tn(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out,
     const uint64_t items4 = (uint64_t)((n + sp_tok_item(4) - 1) / sp_tok_item(4)) * col_tiles;
     const uint64_t items2 = (uint64_t)((n + sp_tok_item(2) - 1) / sp_tok_item(2)) * col_tiles;
     const uint64_t slots = 2ull * ctx->prop.multiProcessorCount;
-    const bool small_items = items4 < slots || 10 * ((items2 + slots - 1) / slots) < 17 * ((items4 + slots - 1) / slots);
+    bool small_items = items4 < slots || 10 * ((items2 + slots - 1) / slots) < 17 * ((items4 + slots - 1) / slots);
+    if (a.g.tune_token_item) small_items = a.g.tune_token_item == 128;
     constexpr int GSB = TN <= 4 ? 32 : 16;  // 32-codebook slices in two buffers where two workgroups still fit a CU
     if constexpr (GSB != 16) {
-        if (a.g.CB_pad % GSB == 0) {
+        if (a.g.CB_pad % GSB == 0 && a.g.tune_cb_per_slice != 16) {
             if (small_items) return launch_sparse_tm<TN, 2, GSB>(ctx, a, d_idx, d_out, d_acc, n, ep);
             return launch_sparse_tm<TN, 4, GSB>(ctx, a, d_idx, d_out, d_acc, n, ep);
         }

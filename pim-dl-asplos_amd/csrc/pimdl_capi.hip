@@ -311,11 +311,49 @@ int pimdl_synchronize(pimdl_ctx* ctx)
 int pimdl_amm_create(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const float* centroids, const void* lut,
                      const float* scales, const float* bias, pimdl_amm** out)
 {
-    return pimdl_amm_create_tuned(ctx, desc, centroids, lut, scales, bias, 0, out);
+    return pimdl_amm_create_with(ctx, desc, centroids, lut, scales, bias, nullptr, out);
 }
 
 int pimdl_amm_create_tuned(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const float* centroids, const void* lut,
                            const float* scales, const float* bias, uint32_t col_block, pimdl_amm** out)
+{
+    pimdl_amm_tuning t;
+    memset(&t, 0, sizeof(t));
+    t.col_block = col_block;
+    return pimdl_amm_create_with(ctx, desc, centroids, lut, scales, bias, &t, out);
+}
+
+int pimdl_amm_set_tuning(pimdl_amm* a, const pimdl_amm_tuning* t)
+{
+    if (!a) return PIMDL_ERR_INVALID;
+    Ctx* ctx = a->ctx;
+    if (!t) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_set_tuning: null argument");
+    const uint32_t kind = a->g.gather_kind == 0 ? PIMDL_GATHER_ROWS : a->g.gather_kind == 1 ? PIMDL_GATHER_ONEHOT : PIMDL_GATHER_SPARSE;
+    if ((t->col_block && t->col_block != a->g.col_block) || (t->gather_kernel && t->gather_kernel != kind))
+        return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_set_tuning: col_block and gather_kernel fix the resident table; "
+                                                 "create the operator with them (pimdl_amm_create_with)");
+    std::string why;
+    AmmGeom g = a->g;
+    if (!apply_runtime_tuning(&g, *t, &why)) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_set_tuning: %s", why.c_str());
+    a->g = g;
+    return PIMDL_OK;
+}
+
+int pimdl_amm_get_tuning(const pimdl_amm* a, pimdl_amm_tuning* t)
+{
+    if (!a || !t) return PIMDL_ERR_INVALID;
+    t->col_block = a->g.col_block;
+    t->gather_kernel = a->g.gather_kind == 0 ? PIMDL_GATHER_ROWS : a->g.gather_kind == 1 ? PIMDL_GATHER_ONEHOT : PIMDL_GATHER_SPARSE;
+    t->token_item = a->g.tune_token_item;
+    t->cb_per_slice = a->g.tune_cb_per_slice;
+    t->xcd_col_split = a->g.tune_xcd_col_split;
+    t->search_kernel = a->g.tune_search;
+    t->search_token_tile = a->g.tune_search_tile;
+    return PIMDL_OK;
+}
+
+int pimdl_amm_create_with(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const float* centroids, const void* lut,
+                          const float* scales, const float* bias, const pimdl_amm_tuning* tuning, pimdl_amm** out)
 {
     if (!ctx) return PIMDL_ERR_INVALID;
     if (!desc || !centroids || !lut || !out) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_create: null argument");
@@ -331,7 +369,7 @@ int pimdl_amm_create_tuned(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const flo
     AmmGeom g;
     memset(&g, 0, sizeof(g));
     std::string why;
-    if (!plan_geometry(plan, ctx->prop.multiProcessorCount, &g, &why, col_block)) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_create: %s", why.c_str());
+    if (!plan_geometry(plan, ctx->prop.multiProcessorCount, &g, &why, tuning)) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_create: %s", why.c_str());
     if (i8_in && !scales) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_create: int8 LUT needs scales");
     if (grouped && desc->lut_bias != 0.0f)
         return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_create: scale_group > 0 has no zero point: lut_bias must be 0");
@@ -399,6 +437,20 @@ int pimdl_amm_create_tuned(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const flo
     }
     *out = a;
     return PIMDL_OK;
+}
+
+int pimdl_amm_set_bias(pimdl_amm* a, const float* bias)
+{
+    if (!a) return PIMDL_ERR_INVALID;
+    Ctx* ctx = a->ctx;
+    int rc = activate(ctx);
+    if (rc) return rc;
+    const size_t bytes = (size_t)a->g.M * sizeof(float);
+    // ordered on the context's stream behind the launches that still read the old values
+    if (bias) rc = hip_check(ctx, hipMemcpyAsync(a->d_bias, bias, bytes, hipMemcpyHostToDevice, ctx->stream), "H2D bias");
+    else rc = hip_check(ctx, hipMemsetAsync(a->d_bias, 0, bytes, ctx->stream), "clear bias");
+    if (rc) return rc;
+    return hip_check(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");  // `bias` may be reused on return
 }
 
 int pimdl_amm_destroy(pimdl_amm* a)
@@ -785,6 +837,24 @@ int pimdl_lut_gather_tiled(pimdl_amm* a, const uint16_t* idx, uint32_t n, float*
     pimdl_tiling til;
     bool ident;
     if ((rc = resolve_tiling(ctx, g, n, tiling, &til, &ident))) return rc;
+    // Every entry must be a centroid id.  The kernels index LDS tables with it, and a buffer that pim_lut has
+    // already rewritten in place (pim_lut_host.cpp:40-104 turns ids into table offsets) would otherwise be
+    // gathered from rows of other codebooks without any error.
+    {
+        const size_t count = (size_t)n * g.CB;
+        uint32_t worst = 0;
+        for (size_t i = 0; i < count; ++i) worst = idx[i] > worst ? idx[i] : worst;
+        if (worst >= g.C) {
+            size_t i = 0;
+            while (idx[i] < g.C) ++i;
+            const size_t ns = til.n_stile_size, cm = til.cb_mtile_size;
+            const size_t in_stile = i % (ns * g.CB), in_mtile = in_stile % (ns * cm);
+            const size_t tok = i / (ns * g.CB) * ns + in_mtile / cm, cb = in_stile / (ns * cm) * cm + in_mtile % cm;
+            return set_error(ctx, PIMDL_ERR_INVALID,
+                             "index buffer entry %zu (token %zu, codebook %zu) is %u: not a centroid id below num_centroid = %u",
+                             i, tok, cb, (unsigned)idx[i], g.C);
+        }
+    }
     if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, idx_buffer_bytes(g, n), "hipMalloc(index scratch)"))) return rc;
     if ((rc = ensure(ctx, &ctx->d_idx16, &ctx->idx16_bytes, (size_t)n * g.CB * 2, "hipMalloc(idx16 scratch)"))) return rc;
     if ((rc = hip_check(ctx, hipMemcpyAsync(ctx->d_idx16, idx, (size_t)n * g.CB * 2, hipMemcpyHostToDevice, ctx->stream), "H2D idx"))) return rc;

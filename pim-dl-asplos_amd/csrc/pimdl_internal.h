@@ -43,6 +43,8 @@ struct AmmGeom {
     uint32_t gather_threads, tokens_per_wg, gather_lds_bytes;
     // ccs kernel
     uint32_t ccs_row_floats, ccs_cb_per_wg, ccs_lds_bytes;
+    // choices a caller has taken over from the library (pimdl_amm_tuning; 0 = the library decides)
+    uint32_t tune_search, tune_search_tile, tune_token_item, tune_cb_per_slice, tune_xcd_col_split;
 };
 
 // fp32 tables whose rows are read in 8-byte chunks (see gather_f32_kernel)
@@ -153,9 +155,10 @@ bool gather_dense_only();
 
 uint32_t ccs_cb_per_wg(uint32_t v);  // codebooks one ccs workgroup covers (0: generic kernel)
 bool gather_rows_only();
-// col_block_hint: 0 = choose the column tile by load balance, else the width to use (an error if this
-// operator's kernel has no such variant)
+// tuning: choices taken over by the caller (nullptr: none); an error if the shape has no kernel for one
 bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::string* why,
-                   uint32_t col_block_hint = 0);
+                   const pimdl_amm_tuning* tuning = nullptr);
+// checks the run-time fields of a tuning against a planned geometry and stores them in it
+bool apply_runtime_tuning(AmmGeom* g, const pimdl_amm_tuning& t, std::string* why);
 
 }  // namespace pimdl

@@ -2,6 +2,15 @@
 // (what `python run_amm.py --amm_config_file X.yaml` ends up running).
 //
 //   test_amm <kernel_config.yaml> [dpu_binary_path (ignored)] [--dump FILE] [--rounds WARMUP RECORD]
+//            [--split] [--load-type 0|1|2] [--refill]
+//
+//   --split      every round calls index_calculation() and then pim_lut() (the two halves amm_host is made of,
+//                amm_host.cpp:10-30) instead of amm_host(); the dump then also holds the index buffer as
+//                pim_lut leaves it (rewritten in place, pim_lut_host.cpp:40-104)
+//   --load-type  overrides kernel_params.lut_load_type (0 static, 1 fine grain, 2 coarse grain)
+//   --refill     before the last round the bias, one LUT entry per row and one centroid are changed IN PLACE
+//                (same buffers, same pointers), as a caller of the reference may do between calls; the dump
+//                holds the changed inputs, so its output must be the one they give
 //
 // Reads the reference's YAML keys (src/host/parser.cpp:22-47): amm_shape_params.{num_codebook,
 // num_centroid, n, input_feature_len, output_feature_len, scale, bias}, system_params.{num_threads,
@@ -16,6 +25,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
 #include <chrono>
 #include <fstream>
 #include <iostream>
@@ -156,13 +166,19 @@ static double now_s()
 int main(int argc, char** argv)
 {
     if (argc < 2) {
-        printf("usage: %s kernel_config_yaml_path [dpu_binary_path] [--dump FILE] [--rounds WARMUP RECORD]\n", argv[0]);
+        printf("usage: %s kernel_config_yaml_path [dpu_binary_path] [--dump FILE] [--rounds WARMUP RECORD] [--split] "
+               "[--load-type T] [--refill]\n", argv[0]);
         return -1;
     }
     string dump_path;
     int warmup = 10, record = 20;  // test_amm.cpp:21-22
+    bool split = false, refill = false;
+    int load_type = -1;
     for (int i = 2; i < argc; ++i) {
         if (!strcmp(argv[i], "--dump") && i + 1 < argc) dump_path = argv[++i];
+        else if (!strcmp(argv[i], "--split")) split = true;
+        else if (!strcmp(argv[i], "--refill")) refill = true;
+        else if (!strcmp(argv[i], "--load-type") && i + 1 < argc) load_type = atoi(argv[++i]);
         else if (!strcmp(argv[i], "--rounds") && i + 2 < argc) {
             warmup = atoi(argv[++i]);
             record = atoi(argv[++i]);
@@ -171,6 +187,7 @@ int main(int argc, char** argv)
     AMMParams amm;
     uint32_t nr_tasklets;
     if (!parse_amm_configs(amm, argv[1], &nr_tasklets)) return -1;
+    if (load_type >= 0) amm.lut_params.lut_load_type = LUTLoadType(load_type);
     const IndexCalcParams& ip = amm.index_params;
     const LUTParams& lp = amm.lut_params;
 
@@ -210,11 +227,30 @@ int main(int argc, char** argv)
     load_binary(&dpu_set, argc > 2 && argv[2][0] != '-' ? argv[2] : "");
     cout << "binary load time is " << now_s() - t1 << endl;
 
+    vector<index_data_type> index_buffer(split ? (size_t)ip.n * ip.num_codebook : 0);
     double total = 0.0;
     for (int round = 0; round < warmup + record; ++round) {
         cout << "---------- ROUND " << round << " ----------" << endl;
+        if (refill && round + 1 == warmup + record && round > 0) {
+            for (auto& b : bias) b = -0.5f * b + 1.0f;
+            // one entry per table row; the DPU-ordered copy is what the call reads
+            for (size_t row = 0; row < (size_t)lp.num_codebook * lp.num_centroid; ++row) {
+                lut_data_type& e = cpu_lut[row * lp.output_feature_len + (row * 7 + 3) % lp.output_feature_len];
+                e = (lut_data_type)(e == 127 ? -128 : e + 1);
+            }
+            to_dpu_lut_order(cpu_lut, dpu_lut, lp);
+            centroids[centroids.size() / 2] += 3.0f;
+            cout << "inputs changed in place" << endl;
+        }
         t1 = now_s();
-        amm_host(&dpu_set, input.data(), centroids.data(), dpu_lut.data(), bias.data(), output.data(), ip, lp);
+        if (split) {
+            // amm_host.cpp:19-29: a zeroed index buffer, index_calculation, pim_lut
+            fill(index_buffer.begin(), index_buffer.end(), (index_data_type)0);
+            index_calculation(input.data(), centroids.data(), index_buffer.data(), ip);
+            pim_lut(lp, &dpu_set, index_buffer.data(), dpu_lut.data(), bias.data(), output.data());
+        } else {
+            amm_host(&dpu_set, input.data(), centroids.data(), dpu_lut.data(), bias.data(), output.data(), ip, lp);
+        }
         double dt = now_s() - t1;
         cout << "PIM AMM time " << dt << endl;
         if (round >= warmup) total += dt;
@@ -239,6 +275,7 @@ int main(int argc, char** argv)
         fwrite(cpu_lut.data(), 1, cpu_lut.size(), fp);
         fwrite(bias.data(), 4, bias.size(), fp);
         fwrite(output.data(), 4, output.size(), fp);
+        if (split) fwrite(index_buffer.data(), sizeof(index_data_type), index_buffer.size(), fp);
         fclose(fp);
         cout << "dumped to " << dump_path << endl;
     }

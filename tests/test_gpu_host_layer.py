@@ -54,28 +54,95 @@ def read_dump(path):
     lut = take(CB * C * M, np.int8).reshape(CB, C, M)
     bias = take(M, np.float32)
     out = take(N * M, np.float32)
+    idx = take(N * CB, np.uint16) if off < len(raw) else None  # --split: the index buffer as pim_lut left it
     assert off == len(raw)
     return dict(N=N, K=K, v=v, C=C, M=M, ns=ns, cm=cm, fs=fs, fm=fm, scale=scale, lut_bias=lut_bias, x=x, cent=cent,
-                lut=lut, bias=bias, out=out)
+                lut=lut, bias=bias, out=out, idx=idx, load_type=load_type, fl=fl, cl=cl)
 
 
-def test_cli_driver_with_reference_yaml_and_dpu_tiling(tmp_path):
-    """`test_amm config.yaml` as run_amm.py would launch it; the output buffer is in DPU order."""
+def run_cli(tmp_path, *flags):
     assert os.path.exists(CLI), "CLI not built (run __graft_entry__.build())"
     dump = str(tmp_path / "dump.bin")
     cfg = os.path.join(ROOT, "tests", "golden", "amm_small_tiled.yaml")
-    res = subprocess.run([CLI, cfg, "ignored_dpu_binary", "--dump", dump, "--rounds", "1", "2"], capture_output=True,
-                         text=True, timeout=120)
+    res = subprocess.run([CLI, cfg, "ignored_dpu_binary", "--dump", dump, *flags], capture_output=True, text=True,
+                         timeout=120)
     assert res.returncode == 0, res.stdout + res.stderr
-    assert "PIM AVG AMM time" in res.stdout and res.stdout.count("PIM AMM time") == 3
-    d = read_dump(dump)
+    return res.stdout, read_dump(dump)
+
+
+def expected_tiled_output(d):
     CB = d["K"] // d["v"]
     idx = oracle.index_calculation(d["x"], d["cent"], d["v"], threads=THREADS)
     acc = oracle.gather_i8(idx, d["lut"], threads=THREADS)
     # the host layer follows pim_lut's epilogue (bias * num_codebook, pim_lut_host.cpp:201)
     want = oracle.dequant(acc, d["bias"], CB, d["scale"], d["lut_bias"], 1, threads=THREADS)
-    want_tiled = tiled_view(want, d["ns"], d["fs"], d["fm"])
-    assert np.array_equal(d["out"].view(np.uint32), want_tiled.view(np.uint32))
+    return tiled_view(want, d["ns"], d["fs"], d["fm"])
+
+
+def test_cli_driver_with_reference_yaml_and_dpu_tiling(tmp_path):
+    """`test_amm config.yaml` as run_amm.py would launch it; the output buffer is in DPU order."""
+    stdout, d = run_cli(tmp_path, "--rounds", "1", "2")
+    assert "PIM AVG AMM time" in stdout and stdout.count("PIM AMM time") == 3
+    assert np.array_equal(d["out"].view(np.uint32), expected_tiled_output(d).view(np.uint32))
+
+
+@pytest.mark.parametrize("load_type", [0, 1, 2])
+def test_index_calculation_then_pim_lut(tmp_path, load_type):
+    """The two halves of amm_host called one after the other through their C++ signatures
+    (index_calc_host.h:5, pim_lut_host.h:13-14) with a non-identity DPU tiling, for the static, fine-grain and
+    coarse-grain LUT orders: the output, and the index buffer as pim_lut leaves it (pim_lut_host.cpp:40-104)."""
+    stdout, d = run_cli(tmp_path, "--split", "--load-type", str(load_type), "--rounds", "1", "1")
+    assert d["load_type"] == load_type and d["idx"] is not None
+    assert np.array_equal(d["out"].view(np.uint32), expected_tiled_output(d).view(np.uint32))
+    CB = d["K"] // d["v"]
+    ids = oracle.index_calculation(d["x"], d["cent"], d["v"], d["ns"], d["cm"], threads=THREADS)
+    want_idx = oracle.prepare_input_index(ids, d["N"], CB, d["C"], d["ns"], d["cm"], load_type, d["fs"], d["fl"], d["cl"])
+    assert np.array_equal(d["idx"], want_idx)
+    assert not np.array_equal(want_idx, np.asarray(ids).reshape(-1))  # the rewrite changed something
+
+
+@pytest.mark.parametrize("flags", [(), ("--split",)])
+def test_inputs_changed_in_place_between_calls(tmp_path, flags):
+    """bias, LUT entries and a centroid change behind the same pointers before the last call; the reference reads
+    all of them anew on every call (pim_lut_host.cpp:143,201), so the last output must follow the new values."""
+    stdout, d = run_cli(tmp_path, "--refill", "--rounds", "1", "2", *flags)
+    assert "inputs changed in place" in stdout
+    assert np.array_equal(d["out"].view(np.uint32), expected_tiled_output(d).view(np.uint32))
+
+
+def test_index_ids_out_of_range_are_refused(ctx):
+    rng = np.random.default_rng(5)
+    N, CB, C, M = 40, 6, 12, 32
+    lut = rng.integers(-128, 128, (CB, C, M)).astype(np.int8)
+    amm = ctx.amm(np.zeros((CB, C, 2), np.float32), lut, np.float32(1.0), None, max_n=N)
+    idx = rng.integers(0, C, (N, CB)).astype(np.uint16)
+    want = oracle.dequant(oracle.gather_i8(idx, lut), np.zeros(M, np.float32), CB, 1.0, 0.0, 0)
+    assert np.array_equal(amm.lut_gather(idx), want)
+    bad = idx.copy()
+    bad[17, 4] = C  # the first id that is not a centroid
+    with pytest.raises(pimdl.PimdlError, match=r"token 17, codebook 4"):
+        amm.lut_gather(bad)
+    # a buffer already rewritten into table offsets, handed in again
+    with pytest.raises(pimdl.PimdlError, match="not a centroid id"):
+        amm.lut_gather(idx * np.uint16(M))
+    amm.close()
+
+
+def test_set_bias(ctx):
+    rng = np.random.default_rng(6)
+    N, K, v, C, M = 70, 32, 4, 16, 50
+    CB = K // v
+    x = rng.standard_normal((N, K)).astype(np.float32)
+    cent = rng.standard_normal((CB, C, v)).astype(np.float32)
+    lut = rng.integers(-128, 128, (CB, C, M)).astype(np.int8)
+    b1, b2 = rng.standard_normal(M).astype(np.float32), rng.standard_normal(M).astype(np.float32)
+    amm = ctx.amm(cent, lut, np.float32(0.3), b1, max_n=N)
+    for step, b in enumerate((b1, b2, None, b1)):
+        if step:
+            amm.set_bias(b)
+        want, _, _ = oracle.amm_cpu(x, cent, lut, np.zeros(M, np.float32) if b is None else b, v, 0.3, 0.0)
+        assert np.array_equal(amm.run(x).view(np.uint32), want.view(np.uint32))
+    amm.close()
 
 
 def test_tiled_entry_points_through_the_c_abi(ctx):

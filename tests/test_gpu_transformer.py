@@ -344,13 +344,73 @@ def test_column_tile_hint_and_measured_tile_search(ctx, tmp_path):
     with pytest.raises(pimdl.PimdlError) as e:
         ctx.amm(cent, lut, np.float32(0.02), None, max_n=N, col_block=80)
     assert e.value.code == pimdl.ERR_INVALID
-    best, results = AT.tune(ctx, pimdl, 512, 128, 4, 16, 384, iters=3)
-    assert best in (48, 64, 96) and best in results and results[best]["gather_ms"] > 0
+    best, results = AT.tune(ctx, pimdl, 512, 128, 4, 16, 384, iters=3, full=False)
+    assert best["gather_ms"] > 0 and best["gather_ms"] <= best["library_gather_ms"] and best["search"] == {}
+    assert {"gather:col_block=48", "gather:col_block=64", "gather:col_block=96"} <= set(results)
     cache = AT.TileCache(str(tmp_path / "tiles.json"))
     key = AT.shape_key("dev", 512, 128, 4, 16, 384, "int8")
     cache.put(key, best)
-    assert AT.TileCache(str(tmp_path / "tiles.json")).get(key) == best
-    AT.write_yaml(str(tmp_path / "t.yaml"), 512, 128, 4, 16, 384, best, results[best])
+    assert AT.TileCache(str(tmp_path / "tiles.json")).get(key) == best["gather"]
+    AT.write_yaml(str(tmp_path / "t.yaml"), 512, 128, 4, 16, 384, best)
     import yaml
     doc = yaml.safe_load(open(str(tmp_path / "t.yaml")))
-    assert doc["amm_shape_params"]["num_codebook"] == 32 and doc["kernel_params"]["col_block"] == best
+    assert doc["amm_shape_params"]["num_codebook"] == 32 and doc["kernel_params"]["gather_ms"] > 0
+
+
+def test_every_tuning_choice_gives_the_same_bits(ctx):
+    """The whole space the measured search walks (accumulation kernel, column block, token item, codebook
+    slice, XCD dealing, search kernel and its token tile): bit-identical outputs, checked against the oracle
+    once; choices a shape has no kernel for are refused with PIMDL_ERR_INVALID."""
+    import itertools
+    rng = np.random.default_rng(3)
+    N, K, v, C, M = 700, 256, 4, 16, 384      # CB = 64: 32-codebook slices exist; 8 | column tiles of 48
+    CB = K // v
+    x = rng.standard_normal((N, K)).astype(np.float32)
+    cent = rng.standard_normal((CB, C, v)).astype(np.float32)
+    lut = rng.integers(-128, 128, (CB, C, M)).astype(np.int8)
+    bias = rng.standard_normal(M).astype(np.float32)
+    want, _, _ = oracle.amm_cpu(x, cent, lut, bias, v, 0.02, 0.0, threads=8)
+    seen = 0
+    for gk, cb in itertools.product((pimdl.GATHER_ROWS, pimdl.GATHER_ONEHOT, pimdl.GATHER_SPARSE), (48, 64, 96)):
+        try:
+            amm = ctx.amm(cent, lut, np.float32(0.02), bias, max_n=N, tuning={"gather_kernel": gk, "col_block": cb})
+        except pimdl.PimdlError as e:
+            assert e.code == pimdl.ERR_INVALID and gk == pimdl.GATHER_ROWS and cb == 96
+            continue
+        assert amm.tuning()["gather_kernel"] == gk and amm.tuning()["col_block"] == cb
+        settings = [{}]
+        if gk != pimdl.GATHER_ROWS:
+            settings += [{"token_item": t} for t in (128, 256)] + [{"xcd_col_split": s} for s in (1, 2, 4, 8, pimdl.XCD_PLAIN)]
+            settings += [{"cb_per_slice": 16}, {"token_item": 128, "cb_per_slice": 16, "xcd_col_split": 2}]
+            if cb <= 64:
+                settings.append({"cb_per_slice": 32})
+        settings += [{"search_kernel": k} for k in (1, 2, 3)] + [{"search_kernel": 3, "search_token_tile": t} for t in (64, 128)]
+        for st in settings:
+            amm.set_tuning(**st)
+            got = amm.run(x)
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (gk, cb, st)
+            seen += 1
+        if gk != pimdl.GATHER_ROWS and cb == 96:
+            with pytest.raises(pimdl.PimdlError):
+                amm.set_tuning(cb_per_slice=32)
+        with pytest.raises(pimdl.PimdlError):
+            amm.set_tuning(col_block=48 if cb != 48 else 64)
+        with pytest.raises(pimdl.PimdlError):
+            amm.set_tuning(token_item=100)
+        amm.close()
+    assert seen > 100
+    # more than 16 centroids: only the byte adder, and no fp32 matrix-core search
+    lut32 = rng.integers(-128, 128, (CB, 32, M)).astype(np.int8)
+    cent32 = rng.standard_normal((CB, 32, v)).astype(np.float32)
+    for bad in ({"gather_kernel": pimdl.GATHER_SPARSE}, {"gather_kernel": pimdl.GATHER_ONEHOT}, {"search_kernel": 2},
+                {"token_item": 128}):
+        with pytest.raises(pimdl.PimdlError) as e:
+            ctx.amm(cent32, lut32, np.float32(0.02), None, max_n=N, tuning=bad)
+        assert e.value.code == pimdl.ERR_INVALID
+
+
+def test_full_measured_search_runs(ctx):
+    from pim_dl_asplos_amd import autotune as AT
+    best, results = AT.tune(ctx, pimdl, 1024, 256, 4, 16, 384, iters=2, full=True)
+    assert any(k.startswith("search:") for k in results) and sum(k.startswith("gather:") for k in results) > 20
+    assert best["gather_ms"] <= best["library_gather_ms"] and best["ccs_ms"] <= best["library_ccs_ms"]
