@@ -290,6 +290,20 @@ PIMDL_API int pimdl_lutgen(pimdl_ctx* ctx, const float* centroids, const float* 
                            uint32_t output_feature_len, uint32_t lut_dtype, uint32_t scale_group,
                            void* lut_out, float* scales_out);
 
+/* The same with the summation order of the product chosen by the caller:
+ *   PIMDL_LUTGEN_MFMA     matrix instruction (what pimdl_lutgen does): the v products of an entry are added
+ *                         in the matrix core's order; entries are within 1e-5 relative of any other order,
+ *                         int8 tables within one quantisation step
+ *   PIMDL_LUTGEN_ORDERED  ascending over the sub-vector from 0.0f, every multiplication and addition rounded
+ *                         on its own: the result of a plain scalar loop, reproducible bit for bit on a CPU
+ *                         (the reference's torch.bmm, pim_weight_converter.py:86-90, fixes no order).
+ * Both read W once and write the table once; the work is memory bound either way. */
+typedef enum pimdl_lutgen_order { PIMDL_LUTGEN_MFMA = 0, PIMDL_LUTGEN_ORDERED = 1 } pimdl_lutgen_order;
+PIMDL_API int pimdl_lutgen_mode(pimdl_ctx* ctx, const float* centroids, const float* weight,
+                                uint32_t num_codebook, uint32_t num_centroid, uint32_t sub_vec_len,
+                                uint32_t output_feature_len, uint32_t lut_dtype, uint32_t scale_group,
+                                uint32_t mode, void* lut_out, float* scales_out);
+
 /* ---- layer normalisation of the transformer layer ---------------------------------------------
  * Replaces norm() (src/host/transformer_layer.cpp:50-90) and, when `residual` is not NULL, the
  * residual add that follows it in the layer (:476-486, :601-611):
@@ -340,6 +354,12 @@ PIMDL_API int pimdl_diag_bandwidth(pimdl_ctx* ctx, uint64_t bytes, float* copy_g
  * search kernel's margin allows 51 of these units (sub_vec_len 4); index_calculation itself
  * (src/host/index_calc_host.cpp:8-53) has no counterpart of this: it is a property of this port. */
 PIMDL_API int pimdl_diag_mfma_error(pimdl_ctx* ctx, uint32_t trials, float* max_err_u);
+/* The same measurement on operands built to make an accumulator lose as much as it can, instead of random
+ * ones: an accumulator of 1.0 that receives 48 equal products just below or just above 1/2, 1 and 2 units in its
+ * last place, of either sign (an adder that rounds to nearest after every product drops all of the first kind,
+ * 24 units in all; one that truncates would drop up to 96), and products that fall by a factor of four from
+ * slot to slot (bits shifted out when the terms of one instruction are aligned).  The margin allows 51. */
+PIMDL_API int pimdl_diag_mfma_error_crafted(pimdl_ctx* ctx, float* max_err_u);
 
 #ifdef __cplusplus
 }

@@ -32,7 +32,7 @@ EXPORTS = ["pimdl_init", "pimdl_destroy", "pimdl_last_error", "pimdl_set_stream"
            "pimdl_layer_norm", "pimdl_get_device_info", "pimdl_amm_get_geometry", "pimdl_diag_bandwidth",
            "pimdl_diag_mfma_error", "pimdl_amm_group_create", "pimdl_amm_group_run", "pimdl_amm_group_destroy",
            "pimdl_attention", "pimdl_amm_group_fused_cols", "pimdl_amm_group_run_fused", "pimdl_amm_run_noalloc", "pimdl_amm_set_bias",
-           "pimdl_amm_create_with", "pimdl_amm_set_tuning", "pimdl_amm_get_tuning"]
+           "pimdl_amm_create_with", "pimdl_amm_set_tuning", "pimdl_amm_get_tuning", "pimdl_lutgen_mode"]
 NOALLOC_SCRATCH_BYTES = 8 << 20
 
 
@@ -217,6 +217,12 @@ class Context:
         self._check(lib().pimdl_diag_mfma_error(self._h, trials, ctypes.byref(e)))
         return e.value
 
+    def diag_mfma_error_crafted(self):
+        """The same on operands built to make the accumulation lose as much as it can (see pimdl.h)."""
+        e = ctypes.c_float(0)
+        self._check(lib().pimdl_diag_mfma_error_crafted(self._h, ctypes.byref(e)))
+        return e.value
+
     def index_calculation(self, x, centroids, n_stile=0, cb_mtile=0):
         """Context-level closest-centroid search: centroids are passed (and uploaded) per call."""
         x = np.ascontiguousarray(x, np.float32)
@@ -228,8 +234,10 @@ class Context:
                                                   cb_mtile))
         return idx.reshape(n, CB) if (n_stile in (0, n) and cb_mtile in (0, CB)) else idx
 
-    def lutgen(self, centroids, weight, lut_dtype=LUT_I8, scale_group=0):
-        """centroids f32 [CB][C][v], weight f32 [K][M] -> (lut [CB][C][M], scales or None)."""
+    def lutgen(self, centroids, weight, lut_dtype=LUT_I8, scale_group=0, ordered=False):
+        """centroids f32 [CB][C][v], weight f32 [K][M] -> (lut [CB][C][M], scales or None).
+        ordered: add the products of an entry in ascending order with separately rounded operations (bit for
+        bit what a scalar loop gives) instead of on the matrix instruction."""
         centroids = np.ascontiguousarray(centroids, np.float32)
         weight = np.ascontiguousarray(weight, np.float32)
         CB, C, v = centroids.shape
@@ -241,8 +249,8 @@ class Context:
         else:
             out = np.empty((CB, C, M), np.int8)
             scales = np.empty(1 if scale_group == 0 else (CB + scale_group - 1) // scale_group, np.float32)
-        self._check(lib().pimdl_lutgen(self._h, _ptr(centroids), _ptr(weight), CB, C, v, M, lut_dtype, scale_group,
-                                       _ptr(out), _ptr(scales)))
+        self._check(lib().pimdl_lutgen_mode(self._h, _ptr(centroids), _ptr(weight), CB, C, v, M, lut_dtype, scale_group,
+                                            1 if ordered else 0, _ptr(out), _ptr(scales)))
         return out, scales
 
     def layer_norm(self, x, weight, bias, residual=None, out=None, eps=1e-6):

@@ -26,6 +26,9 @@ def parse_args(argv=None):
     parser.add_argument("--weight_output_file", type=str, required=True)
     parser.add_argument("--lut_dtype", choices=("int8", "fp32"), default="int8",
                         help="fp32 keeps the unquantised table (scale 1, bias 0); not in the reference")
+    parser.add_argument("--ordered_sum", action="store_true",
+                        help="add the products of a table entry in ascending order with separately rounded fp32 "
+                             "operations (bit for bit a scalar CPU loop) instead of on the matrix instruction")
     return parser.parse_args(argv)
 
 
@@ -66,7 +69,8 @@ def linear_shape(op_name, features):
     return in_features, out_features
 
 
-def convert(tensors, ctx, pimdl, features=768, ncentroids=16, vec_len=2, nsharecodebook=1, lut_dtype="int8"):
+def convert(tensors, ctx, pimdl, features=768, ncentroids=16, vec_len=2, nsharecodebook=1, lut_dtype="int8",
+            ordered_sum=False):
     if nsharecodebook != 1:
         raise ValueError("nsharecodebook != 1 is not supported (the inference engine has one codebook per sub-vector)")
     layers = split_layers(tensors)
@@ -83,10 +87,10 @@ def convert(tensors, ctx, pimdl, features=768, ncentroids=16, vec_len=2, nsharec
             W = np.ascontiguousarray(W, np.float32).reshape(in_f, out_f)
             cent3 = np.ascontiguousarray(cent, np.float32).reshape(CB, ncentroids, vec_len)
             if lut_dtype == "int8":
-                lut, scales = ctx.lutgen(cent3, W, pimdl.LUT_I8, 0)
+                lut, scales = ctx.lutgen(cent3, W, pimdl.LUT_I8, 0, ordered=ordered_sum)
                 scale = np.float32(scales[0])
             else:
-                lut, _ = ctx.lutgen(cent3, W, pimdl.LUT_F32, 0)
+                lut, _ = ctx.lutgen(cent3, W, pimdl.LUT_F32, 0, ordered=ordered_sum)
                 scale = np.float32(1.0)
             out[op + ".lut.tensor"] = lut.reshape(CB * ncentroids, out_f)
             out[op + ".lut.scale"] = np.asarray(scale, np.float32).reshape(())
@@ -107,7 +111,7 @@ def main(argv=None):
     ctx = pimdl.Context(0)
     try:
         out = convert(read_tensors(args.weight_input_file), ctx, pimdl, args.features, args.ncentroids, args.vec_len,
-                      args.nsharecodebook, args.lut_dtype)
+                      args.nsharecodebook, args.lut_dtype, args.ordered_sum)
     finally:
         ctx.close()
     np.savez(args.weight_output_file, **out)

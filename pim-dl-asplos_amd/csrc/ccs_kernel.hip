@@ -1284,9 +1284,17 @@ __global__ void mfma_error_kernel(const uint4* __restrict__ a, const uint4* __re
 }
 }  // namespace
 
-int launch_diag_mfma_error(Ctx* ctx, uint32_t trials, float* max_err_u)
+// crafted: instead of random operands, chains built to make an accumulator lose as much as it can: an
+// accumulator of 1.0 that receives 48 equal products just below / just above a half, one and two units in its
+// last place (a sequential adder that rounds to nearest drops every product of the first kind, one that
+// truncates also drops the larger ones), of either sign, and products whose magnitudes fall by a factor of
+// four from slot to slot (bits shifted out when the terms of one instruction are aligned).  `trials` is
+// ignored then.
+constexpr uint32_t MFMA_CRAFTED_TRIALS = 14;
+int launch_diag_mfma_error(Ctx* ctx, uint32_t trials, bool crafted, float* max_err_u)
 {
     constexpr int CHAIN = 3;
+    if (crafted) trials = MFMA_CRAFTED_TRIALS;
     if (trials == 0 || trials > 4096) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_diag_mfma_error: trials must be in 1..4096");
     std::vector<uint16_t> A((size_t)trials * CHAIN * 32 * 16), B((size_t)trials * CHAIN * 16 * 32);
     std::vector<float> C((size_t)trials * 1024), D((size_t)trials * 1024);
@@ -1300,7 +1308,21 @@ int launch_diag_mfma_error(Ctx* ctx, uint32_t trials, float* max_err_u)
     auto unif = [&]() { return (float)((double)(next() >> 11) / 9007199254740992.0 * 2.0 - 1.0); };
     auto to_bf16 = [](float f) { uint32_t u; memcpy(&u, &f, 4); return (uint16_t)(u >> 16); };
     auto from_bf16 = [](uint16_t h) { uint32_t u = (uint32_t)h << 16; float f; memcpy(&f, &u, 4); return f; };
-    for (uint32_t t = 0; t < trials; ++t) {
+    for (uint32_t t = 0; crafted && t < trials; ++t) {
+        static const float mags[6] = {0.4921875f, 0.5078125f, 0.9921875f, 1.0078125f, 1.984375f, 2.015625f};  // 8-bit significands
+        const float sign = (t & 1) ? -1.0f : 1.0f;
+        for (int m = 0; m < CHAIN; ++m)
+            for (int r = 0; r < 32; ++r)
+                for (int kk = 0; kk < 16; ++kk) {
+                    // A[r][kk] * B[kk][r]: 2^-12 * (sign * mag * 2^-12) = sign * mag * 2^-24, or the falling staircase
+                    const float a = t < 12 ? ldexpf(1.0f, -12) : 1.0f;
+                    const float b = t < 12 ? sign * ldexpf(mags[t / 2], -12) : sign * ldexpf(1.9921875f, -2 * kk - 1);
+                    A[((size_t)(t * CHAIN + m) * 32 + r) * 16 + kk] = to_bf16(a);
+                    B[((size_t)(t * CHAIN + m) * 16 + kk) * 32 + r] = to_bf16(b);
+                }
+        for (size_t i = 0; i < 1024; ++i) C[(size_t)t * 1024 + i] = 1.0f;
+    }
+    for (uint32_t t = 0; !crafted && t < trials; ++t) {
         const float small = ldexpf(1.0f, (int)(t % 5) * 6 - 24);
         for (size_t i = 0; i < (size_t)CHAIN * 512; ++i) {
             A[(size_t)t * CHAIN * 512 + i] = to_bf16(3.0f * unif() * ((next() & 1) ? 1.0f : small));

@@ -61,6 +61,25 @@ __global__ __launch_bounds__(LG_WAVES * 64) void lutgen_f32_kernel(const float* 
     }
 }
 
+// The same product with the v terms of every entry added in ascending order, each multiplication and each
+// addition rounded on its own, starting from 0.0f: the order in which a plain loop over the sub-vector runs
+// on a CPU.  torch.bmm fixes no order (pim_weight_converter.py:86-90 leaves it to the library), so neither
+// form is "the" reference result; this one makes a converter's output reproducible bit for bit by scalar code.
+// One thread = one output column of one codebook, all C centroids: W is read once, the LUT written once.
+__global__ __launch_bounds__(256) void lutgen_ordered_kernel(const float* __restrict__ cent, const float* __restrict__ W,
+                                                           float* __restrict__ lut, uint32_t C, uint32_t v, uint32_t M)
+{
+    const uint32_t f = blockIdx.x * blockDim.x + threadIdx.x, cb = blockIdx.y;
+    if (f >= M) return;
+    const float* w = W + (size_t)cb * v * M + f;
+    for (uint32_t c = 0; c < C; ++c) {
+        const float* a = cent + ((size_t)cb * C + c) * v;
+        float acc = 0.0f;
+        for (uint32_t t = 0; t < v; ++t) acc = __fadd_rn(acc, __fmul_rn(a[t], w[(size_t)t * M]));
+        lut[((size_t)cb * C + c) * M + f] = acc;
+    }
+}
+
 // max |x| per scale group; non-negative floats order like their bit patterns
 __global__ void absmax_kernel(const float* __restrict__ lut, uint32_t* __restrict__ absmax_bits,
                               uint64_t group_elems, uint64_t total)
@@ -123,8 +142,12 @@ __global__ __launch_bounds__(1024) void lds_read_kernel(int* __restrict__ sink, 
 }  // namespace
 
 int launch_lutgen_f32(Ctx* ctx, const float* d_cent, const float* d_w, float* d_lut, uint32_t CB, uint32_t C,
-                      uint32_t v, uint32_t M)
+                      uint32_t v, uint32_t M, bool ordered)
 {
+    if (ordered) {
+        hipLaunchKernelGGL(lutgen_ordered_kernel, dim3((M + 255) / 256, CB), dim3(256), 0, ctx->stream, d_cent, d_w, d_lut, C, v, M);
+        return hip_check(ctx, hipGetLastError(), "lutgen_ordered_kernel launch");
+    }
     dim3 grid((M + LG_WAVES * 16 * LG_FT - 1) / (LG_WAVES * 16 * LG_FT), (C + 15) / 16, CB);
     hipLaunchKernelGGL(lutgen_f32_kernel, grid, dim3(LG_WAVES * 64), 0, ctx->stream, d_cent, d_w, d_lut, CB, C, v, M);
     return hip_check(ctx, hipGetLastError(), "lutgen_f32_kernel launch");

@@ -870,7 +870,14 @@ int pimdl_lut_gather(pimdl_amm* a, const uint16_t* idx, uint32_t n, float* out)
 int pimdl_lutgen(pimdl_ctx* ctx, const float* centroids, const float* weight, uint32_t CB, uint32_t C, uint32_t v,
                  uint32_t M, uint32_t lut_dtype, uint32_t scale_group, void* lut_out, float* scales_out)
 {
+    return pimdl_lutgen_mode(ctx, centroids, weight, CB, C, v, M, lut_dtype, scale_group, PIMDL_LUTGEN_MFMA, lut_out, scales_out);
+}
+
+int pimdl_lutgen_mode(pimdl_ctx* ctx, const float* centroids, const float* weight, uint32_t CB, uint32_t C, uint32_t v,
+                      uint32_t M, uint32_t lut_dtype, uint32_t scale_group, uint32_t mode, void* lut_out, float* scales_out)
+{
     if (!ctx) return PIMDL_ERR_INVALID;
+    if (mode != PIMDL_LUTGEN_MFMA && mode != PIMDL_LUTGEN_ORDERED) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_lutgen: unknown mode");
     if (!centroids || !weight || !lut_out) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_lutgen: null argument");
     if (!CB || !C || !v || !M) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_lutgen: zero-sized dimension");
     if (lut_dtype != PIMDL_LUT_I8 && lut_dtype != PIMDL_LUT_F32) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_lutgen: unknown lut_dtype");
@@ -887,7 +894,7 @@ int pimdl_lutgen(pimdl_ctx* ctx, const float* centroids, const float* weight, ui
     if (!rc) rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&d_lut), lut_elems * 4), "hipMalloc(lutgen lut)");
     if (!rc) rc = hip_check(ctx, hipMemcpyAsync(d_cent, centroids, cent_bytes, hipMemcpyHostToDevice, ctx->stream), "H2D centroids");
     if (!rc) rc = hip_check(ctx, hipMemcpyAsync(d_w, weight, w_bytes, hipMemcpyHostToDevice, ctx->stream), "H2D weight");
-    if (!rc) rc = launch_lutgen_f32(ctx, d_cent, d_w, d_lut, CB, C, v, M);
+    if (!rc) rc = launch_lutgen_f32(ctx, d_cent, d_w, d_lut, CB, C, v, M, mode == PIMDL_LUTGEN_ORDERED);
     if (!rc && lut_dtype == PIMDL_LUT_F32) {
         rc = hip_check(ctx, hipMemcpyAsync(lut_out, d_lut, lut_elems * 4, hipMemcpyDeviceToHost, ctx->stream), "D2H lut");
     } else if (!rc) {
@@ -1018,7 +1025,16 @@ int pimdl_diag_mfma_error(pimdl_ctx* ctx, uint32_t trials, float* max_err_u)
     if (!max_err_u) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_diag_mfma_error: null result pointer");
     int rc = activate(ctx);
     if (rc) return rc;
-    return launch_diag_mfma_error(ctx, trials, max_err_u);
+    return launch_diag_mfma_error(ctx, trials, false, max_err_u);
+}
+
+int pimdl_diag_mfma_error_crafted(pimdl_ctx* ctx, float* max_err_u)
+{
+    if (!ctx) return PIMDL_ERR_INVALID;
+    if (!max_err_u) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_diag_mfma_error_crafted: null result pointer");
+    int rc = activate(ctx);
+    if (rc) return rc;
+    return launch_diag_mfma_error(ctx, 0, true, max_err_u);
 }
 
 }  // extern "C"

@@ -136,7 +136,7 @@ int launch_pack_idx(Ctx* ctx, const AmmGeom& g, const uint16_t* d_idx16, uint8_t
 int launch_retile_output(Ctx* ctx, const float* d_rowmajor, float* d_tiled, uint32_t n, uint32_t M,
                          uint32_t n_stile, uint32_t f_stile, uint32_t f_mtile);
 int launch_lutgen_f32(Ctx* ctx, const float* d_cent, const float* d_w, float* d_lut, uint32_t CB,
-                      uint32_t C, uint32_t v, uint32_t M);
+                      uint32_t C, uint32_t v, uint32_t M, bool ordered = false);
 int launch_lut_quant(Ctx* ctx, const float* d_lut, int8_t* d_q, float* d_scales, uint32_t CB, uint32_t C,
                      uint32_t M, uint32_t scale_group);
 int launch_layer_norm(Ctx* ctx, const float* d_x, const float* d_w, const float* d_b, const float* d_residual,
@@ -144,7 +144,7 @@ int launch_layer_norm(Ctx* ctx, const float* d_x, const float* d_w, const float*
 int launch_attention_hd64(Ctx* ctx, const float* d_q, const float* d_k, const float* d_v, float* d_out, uint32_t batch,
                           uint32_t seq, uint32_t heads, uint32_t in_stride, uint32_t out_stride, float scale);
 int launch_diag(Ctx* ctx, uint64_t bytes, float* copy_gbps, float* lds_gbps);
-int launch_diag_mfma_error(Ctx* ctx, uint32_t trials, float* max_err_u);
+int launch_diag_mfma_error(Ctx* ctx, uint32_t trials, bool crafted, float* max_err_u);
 
 // the sparse one-hot gather (gather_sp_kernel.hip)
 int launch_gather_sparse(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_t* d_acc_or_null,

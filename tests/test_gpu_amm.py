@@ -465,6 +465,16 @@ def test_matrix_core_rounding_stays_inside_the_search_margin(ctx):
     assert 0.0 < worst < 12.0, worst
 
 
+def test_matrix_core_rounding_on_crafted_worst_cases(ctx):
+    """Random operands are not the worst case for an accumulator.  The crafted chains add 48 equal products just
+    below / above 1/2, 1 and 2 units in the last place of an accumulator of 1.0 (either sign), and products
+    falling by a factor of four per slot: a sequential round-to-nearest adder loses 24 units on them, a
+    truncating one up to 96.  The search margin allows 51; the device must stay below half of that."""
+    worst = ctx.diag_mfma_error_crafted()
+    print("crafted mfma error (units of 2^-24 * sum|terms|):", worst)
+    assert 0.0 <= worst < 25.5, worst
+
+
 def test_search_at_full_ffn2_shape(ctx):
     """N=8192, K=3072, v=4, 16 centroids: every index of the headline shape against the oracle,
     once with N(0,1) data and once with the reference driver's ranges."""

@@ -72,9 +72,11 @@ def test_vit_base_sweep_full_batch(env, v, C, lut_kind):
     run_and_check_sample(env[1], 13 + v + C, 12608, 768, v, C, 3072, lut_kind, sample=96)
 
 
-@pytest.mark.parametrize("v,C", [(2, 16), (4, 16), (8, 32)])
-def test_vit_base_ffn2_full_batch(env, v, C):
-    run_and_check_sample(env[1], 29 + v, 12608, 3072, v, C, 768, "i8", sample=96)
+@pytest.mark.parametrize("lut_kind", ["i8", "f32"])
+@pytest.mark.parametrize("v,C", [(2, 8), (2, 16), (2, 32), (4, 8), (4, 16), (4, 32), (8, 8), (8, 16), (8, 32)])
+def test_vit_base_ffn2_sweep_full_batch(env, v, C, lut_kind):
+    """The second feed-forward matrix of ViT-Base (3072 -> 768) over the same sweep, both LUT types."""
+    run_and_check_sample(env[1], 29 + v + C, 12608, 3072, v, C, 768, lut_kind, sample=64)
 
 
 def test_reference_single_amm_search_space_shape(env):

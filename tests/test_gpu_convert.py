@@ -42,6 +42,24 @@ def test_lutgen_matches_the_converter_formula(ctx, CB, C, v, M):
     assert np.abs(got_q.astype(np.int32)).max() == 127
 
 
+@pytest.mark.parametrize("CB,C,v,M", [(192, 16, 4, 3072), (384, 16, 2, 768), (96, 32, 8, 200), (7, 5, 3, 33), (1, 1, 1, 4),
+                                      (12, 16, 32, 100)])
+def test_ordered_lutgen_is_bit_identical_to_the_scalar_loop(ctx, CB, C, v, M):
+    """PIMDL_LUTGEN_ORDERED: fp32 table, int8 table and scale(s) equal the oracle's bit for bit."""
+    rng = np.random.default_rng(CB * 7 + C + v + M)
+    cent = rng.standard_normal((CB, C, v)).astype(np.float32)
+    W = (rng.standard_normal((CB * v, M)) * 0.02).astype(np.float32)
+    W[0, :2] = [0.0, -0.0]
+    want_f = oracle.lutgen_f32(cent, W, threads=8)
+    got_f, _ = ctx.lutgen(cent, W, pimdl.LUT_F32, 0, ordered=True)
+    assert np.array_equal(got_f.view(np.uint32), want_f.view(np.uint32))
+    for group in (0, 1, 5):
+        want_q, want_s = oracle.lut_quant(want_f, group)
+        got_q, got_s = ctx.lutgen(cent, W, pimdl.LUT_I8, group, ordered=True)
+        assert np.array_equal(got_s.view(np.uint32), np.asarray(want_s, np.float32).view(np.uint32))
+        assert np.array_equal(got_q, want_q)
+
+
 def test_converter_writes_the_engine_format_and_the_model_runs_from_it(ctx, tmp_path):
     """A synthetic 'calibrated checkpoint' in the reference's input naming (safetensors, HF BERT encoder keys)
     goes through the converter; the result loads into the model wrapper and runs."""
