@@ -7,7 +7,7 @@ reference's per-tensor fp32 scale, int32 accumulation, random-init centroids and
 One "step" = one pass of the pair (centroid search + LUT gather for FFN1, then for FFN2) with all
 inputs, LUTs and outputs resident in HBM.  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-model] [--no-sweep] [--no-cpu-baseline]
 """
 import argparse
 import json
@@ -21,17 +21,18 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0                     # MI355X HBM3E
-# HBM bytes per launch of the gather kernels at this workload, from two rocprofv3 --pmc runs of this
-# script (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch).  FETCH_SIZE is scaled by 2.0 and
-# WRITE_SIZE by 1.0: the factors a streaming kernel of known size gives for the same counters on
-# this part.  Summary: profiles/bench_ffn_pair_hbm_traffic.txt.  Keyed by (K, M).
-MEASURED_GATHER_TRAFFIC = {
-    (768, 3072): {"fetch_kib": 7992.3, "write_kib": 111172.0},
-    (3072, 768): {"fetch_kib": 15578.0, "write_kib": 26636.7},
-}
-FETCH_SCALE, WRITE_SCALE = 2.0, 1.0
 LDS_PEAK_GBPS = 256 * 256 * 2.4            # 256 CUs x 256 B/clk (ds_read_b128) x 2.4 GHz = 157286 GB/s
 MFMA_I8_PEAK_TOPS = 5000.0                 # MI355X dense int8 matrix peak
+# HBM bytes per launch of the dominant gather kernel, from two rocprofv3 --pmc runs of this script
+# (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch; summary: profiles/bench_ffn_pair_hbm_traffic.txt).
+# Keyed by the kernel's name as a profile lists it and by the batch: the figure is only reported while the
+# launch still runs that kernel on that batch, otherwise `traffic` is null until the counters are collected again.
+# FETCH_SIZE is scaled by 2.0 and WRITE_SIZE by 1.0: what a streaming copy of known size reads for the same
+# counters in the same runs.
+MEASURED_GATHER_TRAFFIC = {
+}
+FETCH_SCALE, WRITE_SCALE = 2.0, 1.0
+CLOCK_SETTLE_S = 0.08                      # untimed pre-heat: the engine clock needs ~20 ms of this load to ramp up
 
 
 def synth_amm(rng, K, v, C, M, pimdl, ctx):
@@ -89,50 +90,113 @@ def model_forward(pimdl, ctx, iters=10):
             "note": "LUT-AMM linears (tanh-GELU inside the first feed-forward operator's epilogue), pimdl_layer_norm and pimdl_attention (fp32) on libpimdl; PyTorch-ROCm for tensors, streams and graph capture"}
 
 
-def cpu_baseline(shapes, N, budget_s=12.0):
-    """The oracle's restatement of the reference's amm_cpu (test_amm.cpp:126-183), timed on this
-    host's cores on a bounded token sample of the same two AMMs."""
+def cpu_baseline(shapes, N, warmup=10, rounds=20, budget_s=25.0):
+    """The oracle's restatement of the reference's amm_cpu (test_amm.cpp:126-183) on this host's cores, on the
+    full batch of both AMMs, with the reference driver's protocol (test_amm.cpp:21-22,290-314: 10 warm-up and
+    20 timed rounds, mean wall time).  Bounded: if the first round says the protocol would exceed budget_s, the
+    round counts shrink in proportion (and the sample string says so)."""
     import oracle
 
     threads = oracle.max_threads()
     rng = np.random.default_rng(1)
-    ns = min(N, 1024)
     work = []
     for (K, v, C, M) in shapes:
         CB = K // v
-        x = rng.standard_normal((ns, K)).astype(np.float32)
+        x = rng.standard_normal((N, K), dtype=np.float32)
         cent = rng.standard_normal((CB, C, v)).astype(np.float32)
         lut = rng.integers(-128, 128, (CB, C, M)).astype(np.int8)
         bias = np.zeros(M, np.float32)
-        scratch = (np.empty((ns, CB), np.uint16), np.empty((ns, M), np.int32), np.empty((ns, M), np.float32))
+        scratch = (np.empty((N, CB), np.uint16), np.empty((N, M), np.int32), np.empty((N, M), np.float32))
         work.append((x, cent, lut, bias, v, scratch))
 
     def one_pass():
         for x, cent, lut, bias, v, scratch in work:
             oracle.amm_cpu(x, cent, lut, bias, v, 0.01, 0.0, threads=threads, scratch=scratch)
 
-    one_pass()  # warm-up
     t0 = time.perf_counter()
-    one_pass()
+    one_pass()  # first warm-up round, timed only to bound the rest
     t1 = time.perf_counter() - t0
-    rounds = int(max(2, min(20, budget_s / max(t1, 1e-3))))
+    shrink = min(1.0, budget_s / max(t1 * (warmup + rounds), 1e-9))
+    warmup, rounds = max(1, int(warmup * shrink)), max(2, int(rounds * shrink))
+    for _ in range(warmup - 1):
+        one_pass()
     t0 = time.perf_counter()
     for _ in range(rounds):
         one_pass()
     dt = (time.perf_counter() - t0) / rounds
-    return {"value": ns / dt, "unit": "tokens/s", "cores": threads, "kind": "port",
-            "sample": f"{ns} of {N} tokens through both AMMs of the pair, {rounds} timed rounds after 1 warm-up, "
-                      f"oracle amm_cpu (-O3 -fopenmp, no -march), {dt * 1e3:.1f} ms per round"}
+    eff = sum(2.0 * N * K * M for (K, _, _, M) in shapes)
+    return {"value": N / dt, "unit": "tokens/s", "cores": threads, "kind": "port", "eff_gops": eff / dt / 1e9,
+            "sample": f"all {N} tokens through both AMMs of the pair, {rounds} timed rounds after {warmup} warm-up "
+                      f"(the reference driver's protocol is 20 after 10), oracle amm_cpu built with the reference's "
+                      f"flags (-O3 -fopenmp, no -march), {threads} OpenMP threads, {dt * 1e3:.1f} ms per round"}
+
+
+def per_codebook_scale(pimdl, ctx, rng, N, shapes, iters=20):
+    """The same pair with one fp32 scale per codebook (scale_group = 1), the wording of the benchmark
+    configuration; the reference itself has one scale per tensor, which is what `value` measures.  A different
+    scale per codebook rules out integer accumulation across codebooks: the table is resident as fp32 integers
+    and gathered by the fp32-table kernel (VALU adds), so this mode runs at that kernel's rate."""
+    import torch
+    out = []
+    for (K, v, C, M) in shapes:
+        CB = K // v
+        cent = rng.standard_normal((CB, C, v)).astype(np.float32)
+        W = (rng.standard_normal((K, M)) * 0.02).astype(np.float32)
+        lut, scales = ctx.lutgen(cent, W, pimdl.LUT_I8, 1)
+        amm = ctx.amm(cent, lut, scales, None, max_n=N, scale_group=1)
+        x = torch.randn((N, K), device="cuda", dtype=torch.float32)
+        y = torch.empty((N, M), device="cuda", dtype=torch.float32)
+        t = amm.profile(x.data_ptr(), N, y.data_ptr(), warmup=20, iters=iters)
+        out.append({"K": K, "M": M, "ccs_ms": t["ccs_ms"], "gather_ms": t["gather_ms"], "amm_ms": t["total_ms"],
+                    "gather_kernel": amm.last_gather_kernel()})
+        amm.close()
+    total = sum(o["amm_ms"] for o in out)
+    return {"scale_group": 1, "per_amm": out, "ms_per_step": total, "tokens_per_s": N / (total * 1e-3),
+            "note": "extension (one scale per codebook is not in the reference); int32 sum inside a group, fp32 "
+                    "across groups in ascending order; bit-identical to the oracle's statement of it"}
+
+
+def vit_sweep(pimdl, ctx, iters=10):
+    """ViT-Base/16 feed-forward shapes (N = 64 x 197 = 12608) over sub_vec_len x num_centroid x LUT type:
+    device time of the two kernels of each operator."""
+    import torch
+    N = 64 * 197
+    rng = np.random.default_rng(4)
+    cells = []
+    for (K, M) in ((768, 3072), (3072, 768)):
+        x = torch.randn((N, K), device="cuda", dtype=torch.float32)
+        y = torch.empty((N, M), device="cuda", dtype=torch.float32)
+        for v in (2, 4, 8):
+            for C in (8, 16, 32):
+                CB = K // v
+                cent = rng.standard_normal((CB, C, v)).astype(np.float32)
+                for kind in ("i8", "f32"):
+                    if kind == "i8":
+                        lut, scales = rng.integers(-128, 128, (CB, C, M)).astype(np.int8), np.float32(0.01)
+                    else:
+                        lut, scales = rng.standard_normal((CB, C, M), dtype=np.float32), None
+                    amm = ctx.amm(cent, lut, scales, None, max_n=N)
+                    t = amm.profile(x.data_ptr(), N, y.data_ptr(), warmup=5, iters=iters)
+                    e = 1 if kind == "i8" else 4
+                    cells.append({"K": K, "M": M, "v": v, "C": C, "lut": kind, "ccs_us": round(t["ccs_ms"] * 1e3, 1),
+                                  "gather_us": round(t["gather_ms"] * 1e3, 1),
+                                  "mtok_per_s": round(N / (t["total_ms"] * 1e-3) / 1e6, 1),
+                                  "gather_lds_frac": round(e * N * CB * M / (t["gather_ms"] * 1e-3) / 1e9 / LDS_PEAK_GBPS, 3),
+                                  "gather_kernel": amm.last_gather_kernel().split("<")[0]})
+                    amm.close()
+                    del lut
+    return {"tokens": N, "cells": cells}
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=500)
-    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--tokens", type=int, default=8192)
     ap.add_argument("--no-model", action="store_true", help="skip the 12-layer model forward timing")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the ViT-Base sweep and the per-codebook-scale pair")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (the path shards over tokens with no exchange; "
@@ -174,6 +238,16 @@ def main():
         amms[0].run_ptr(x1.data_ptr(), N, h.data_ptr())
         amms[1].run_ptr(x2.data_ptr(), N, y.data_ptr())
 
+    # Untimed pre-heat, whatever --warmup says: after an idle period the engine clock takes about 20 ms of this
+    # load to ramp up, and until then everything runs 15-20 % slower.  Then the W warm-up steps, then exactly K
+    # timed steps between two synchronisations.
+    settle_steps = 0
+    t_end = time.perf_counter() + CLOCK_SETTLE_S
+    while time.perf_counter() < t_end:
+        for _ in range(50):
+            step()
+        torch.cuda.synchronize()
+        settle_steps += 50
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -188,10 +262,9 @@ def main():
     ev_ms = e0.elapsed_time(e1) / args.steps
     ms_per_step = wall_ms
 
-    # per-kernel device times (HIP events on the same stream, each kernel launched on its own)
-    # (the engine clock takes about a hundred steps to settle after an idle period, hence the warm-up)
-    prof = [amms[0].profile(x1.data_ptr(), N, h.data_ptr(), warmup=max(3, args.warmup), iters=max(10, args.steps)),
-            amms[1].profile(x2.data_ptr(), N, y.data_ptr(), warmup=max(3, args.warmup), iters=max(10, args.steps))]
+    # per-kernel device times: HIP events on the launch stream, each kernel launched on its own (pimdl_amm_profile)
+    prof = [amms[0].profile(x1.data_ptr(), N, h.data_ptr(), warmup=200, iters=max(50, args.steps)),
+            amms[1].profile(x2.data_ptr(), N, y.data_ptr(), warmup=200, iters=max(50, args.steps))]
     per_amm = []
     for name, (K, vv, CC, M), p in zip(("ffn1", "ffn2"), shapes, prof):
         ab = algorithmic_bytes(N, K, vv, CC, M)
@@ -208,41 +281,43 @@ def main():
         })
     for pa, amm in zip(per_amm, amms):
         pa["geometry"] = amm.geometry()
+        pa["gather_kernel"] = amm.last_gather_kernel()
 
-    # dominant kernel: the longer of the two gathers
+    # Dominant kernel: the longer of the two gathers.  Its roofline is the one the metric is worded in: LUT
+    # entries gathered per second, N*CB*M algorithmic bytes per launch, over the LDS read peak.  How the kernel
+    # gets there (one-hot products on the matrix cores, which execute 16 multiply-adds per gathered entry) is
+    # reported beside it as utilisation of the units it occupies, not as a roofline fraction.
     dom = max(per_amm, key=lambda d: d["gather_ms"])
     K, M = dom["K"], dom["M"]
     ab = algorithmic_bytes(N, K, v, C, M)
     _, lds_measured = ctx.diag_bandwidth(copy=False, lds=True)
-    mt = MEASURED_GATHER_TRAFFIC.get((K, M)) if N == 8192 else None
+    mt = MEASURED_GATHER_TRAFFIC.get((dom["gather_kernel"], N, K, M))
     traffic = (mt["fetch_kib"] * FETCH_SCALE + mt["write_kib"] * WRITE_SCALE) * 1024.0 if mt else None
-    # The gather for C <= 16 runs as a one-hot int8 matrix product on the MFMA units: per launch it
-    # executes 2 * N * (CB * 16) * M int8 operations to perform the N * CB * M algorithmic adds.
-    one_hot = C <= 16
-    mfma_ops = 2.0 * N * (K // v) * 16 * M
-    mfma_tops = mfma_ops / (dom["gather_ms"] * 1e-3) / 1e12
+    sparse = dom["gather_kernel"].startswith("gather_sparse")
+    cb_per_instr = 8 if sparse else 4               # codebooks one matrix instruction covers for 16 tokens x 16 columns
+    instrs = N / 16 * (M / 16) * (K // v) / cb_per_instr
+    simds = 4 * ctx.device_info()["compute_units"]
     roofline = {
-        "kernel": f"gather_onehot_kernel ({dom['name']}: K={K} M={M})" if one_hot
-                  else f"gather_i8_kernel ({dom['name']}: K={K} M={M})",
-        "bound": "mfma" if one_hot else "lds",
-        "achieved": mfma_tops if one_hot else dom["gather_lds_gbps"],
-        "peak": MFMA_I8_PEAK_TOPS if one_hot else LDS_PEAK_GBPS,
-        "unit": "TOP/s" if one_hot else "GB/s",
-        "frac": (mfma_tops / MFMA_I8_PEAK_TOPS) if one_hot else dom["gather_lds_frac"],
-        "traffic": traffic,
-        "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this script, scaled x2.0 / x1.0 "
-                          "(copy-kernel calibration); recorded constant, not collected in this run",
-        "executed_int8_ops_per_launch": mfma_ops,
-        "algorithmic_adds_per_launch": ab["gather_lds"],
+        "kernel": f"{dom['gather_kernel']} ({dom['name']}: K={K} M={M})",
+        "bound": "lds",
+        "achieved": dom["gather_lds_gbps"], "peak": LDS_PEAK_GBPS, "unit": "GB/s", "frac": dom["gather_lds_frac"],
+        "algorithmic_bytes_per_launch": ab["gather_lds"],
         "avg_launch_ms": dom["gather_ms"],
-        # the same launch against the LDS-gather roofline the metric is worded in: bytes of LUT
-        # entries gathered per second (N*CB*M bytes per launch) over the LDS read peak
-        "lds": {"achieved": dom["gather_lds_gbps"], "peak": LDS_PEAK_GBPS, "unit": "GB/s",
-                "frac": dom["gather_lds_frac"], "algorithmic_bytes_per_launch": ab["gather_lds"],
-                "lds_peak_measured_gbps": lds_measured,
-                "frac_of_measured_lds_peak": dom["gather_lds_gbps"] / lds_measured if lds_measured else None},
+        "traffic": traffic,
+        "traffic_source": ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this script for this kernel and batch, scaled "
+                           "x2.0 / x1.0 (copy-kernel calibration); profiles/bench_ffn_pair_hbm_traffic.txt") if mt else
+                          "not collected for the kernel this run launched",
+        "lds_peak_measured_gbps": lds_measured,
+        "frac_of_measured_lds_peak": dom["gather_lds_gbps"] / lds_measured if lds_measured else None,
         "hbm": {"achieved": dom["gather_hbm_gbps"], "peak": HBM_PEAK_GBPS, "frac": dom["gather_hbm_frac"],
                 "algorithmic_bytes_per_launch": ab["gather_hbm"]},
+        # utilisation, not a roofline: matrix instructions issued per launch x 16 clocks each over the SIMDs' time
+        "matrix_core": {"instruction": "v_smfmac_i32_16x16x128_i8" if sparse else "v_mfma_i32_16x16x64_i8",
+                        "instructions_per_launch": instrs,
+                        "busy_frac": instrs * 16.0 / (simds * 2.4e9 * dom["gather_ms"] * 1e-3),
+                        "dense_equivalent_tops": 2.0 * N * (K // v) * 16 * M / (dom["gather_ms"] * 1e-3) / 1e12,
+                        "dense_int8_peak_tops": MFMA_I8_PEAK_TOPS},
+        "north_star_target_frac": 0.5,
     }
 
     total_eff_ops = sum(algorithmic_bytes(N, K_, v, C, M_)["eff_ops"] for (K_, _, _, M_) in shapes)
@@ -251,6 +326,7 @@ def main():
         "value": N / (ms_per_step * 1e-3),
         "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "clock_settle_steps": settle_steps,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "i8", "data": "synthetic",
         "config": {"workload": "BERT-base FFN pair as LUT-AMM: N=8192 (64x128) fp32 activations N(0,1); "
@@ -277,6 +353,9 @@ def main():
                               "note": "pageable host memory in and out of both AMMs (PCIe copies included), 3 steps"}
     if not args.no_model:
         result["bert_base_forward"] = model_forward(pimdl, ctx)
+    if not args.no_sweep:
+        result["per_codebook_scale"] = per_codebook_scale(pimdl, ctx, rng, N, shapes)
+        result["vit_base_sweep"] = vit_sweep(pimdl, ctx)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(shapes, N)
     for a in amms:

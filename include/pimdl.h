@@ -344,6 +344,10 @@ typedef struct pimdl_amm_geometry {
     uint32_t ccs_tokens_per_wg, ccs_cb_per_wg, ccs_threads, ccs_lds_bytes;
 } pimdl_amm_geometry;
 PIMDL_API int pimdl_amm_get_geometry(const pimdl_amm* amm, pimdl_amm_geometry* g);
+/* Name, with template arguments, of the gather kernel the operator's last launch used ("" before the first
+ * launch): the name a profile of that launch lists, so that a benchmark can tell which kernel its counters
+ * belong to. */
+PIMDL_API int pimdl_amm_last_gather_kernel(const pimdl_amm* amm, char* name, size_t len);
 /* Achieved bandwidth, GB/s, of (a) a plain device-to-device copy kernel of `bytes` bytes and
  * (b) a ds_read_b128 loop that keeps every CU's LDS busy.  Either pointer may be NULL. */
 PIMDL_API int pimdl_diag_bandwidth(pimdl_ctx* ctx, uint64_t bytes, float* copy_gbps,

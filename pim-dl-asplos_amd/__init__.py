@@ -32,7 +32,8 @@ EXPORTS = ["pimdl_init", "pimdl_destroy", "pimdl_last_error", "pimdl_set_stream"
            "pimdl_layer_norm", "pimdl_get_device_info", "pimdl_amm_get_geometry", "pimdl_diag_bandwidth",
            "pimdl_diag_mfma_error", "pimdl_amm_group_create", "pimdl_amm_group_run", "pimdl_amm_group_destroy",
            "pimdl_attention", "pimdl_amm_group_fused_cols", "pimdl_amm_group_run_fused", "pimdl_amm_run_noalloc", "pimdl_amm_set_bias",
-           "pimdl_amm_create_with", "pimdl_amm_set_tuning", "pimdl_amm_get_tuning", "pimdl_lutgen_mode"]
+           "pimdl_amm_create_with", "pimdl_amm_set_tuning", "pimdl_amm_get_tuning", "pimdl_lutgen_mode",
+           "pimdl_diag_mfma_error_crafted", "pimdl_amm_last_gather_kernel"]
 NOALLOC_SCRATCH_BYTES = 8 << 20
 
 
@@ -156,6 +157,13 @@ def lib():
     for name in EXPORTS:
         if name != "pimdl_last_error":
             getattr(L, name).restype = ctypes.c_int
+    L.pimdl_amm_last_gather_kernel.argtypes = [vp, ctypes.c_char_p, ctypes.c_size_t]
+    L.pimdl_amm_set_bias.argtypes = [vp, vp]
+    L.pimdl_amm_create_with.argtypes = [vp, ctypes.POINTER(AmmDesc), vp, vp, vp, vp, ctypes.POINTER(AmmTuning), ctypes.POINTER(vp)]
+    L.pimdl_amm_set_tuning.argtypes = [vp, ctypes.POINTER(AmmTuning)]
+    L.pimdl_amm_get_tuning.argtypes = [vp, ctypes.POINTER(AmmTuning)]
+    L.pimdl_lutgen_mode.argtypes = [vp, vp, vp, u32, u32, u32, u32, u32, u32, u32, vp, vp]
+    L.pimdl_diag_mfma_error_crafted.argtypes = [vp, ctypes.POINTER(ctypes.c_float)]
     _lib = L
     return L
 
@@ -386,6 +394,12 @@ class Amm:
         g = AmmGeometry()
         self.ctx._check(lib().pimdl_amm_get_geometry(self._h, ctypes.byref(g)))
         return g.asdict()
+
+    def last_gather_kernel(self):
+        """Name (with template arguments) of the gather kernel of the last launch, as a profile lists it."""
+        buf = ctypes.create_string_buffer(96)
+        self.ctx._check(lib().pimdl_amm_last_gather_kernel(self._h, buf, 96))
+        return buf.value.decode()
 
     def run(self, x, out=None):
         """x: numpy f32 [n][K] (host) -> numpy f32 [n][M]."""

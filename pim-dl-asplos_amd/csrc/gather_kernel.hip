@@ -41,6 +41,8 @@
 // (bit-identical to a sequential CPU sum).
 #include <stdlib.h>
 
+#include <stdio.h>
+
 #include "gather_common.h"
 
 namespace pimdl {
@@ -809,6 +811,7 @@ int launch_onehot_tm(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out,
     const XcdMap xmap = choose_xcd_map(a.g.M_pad / (16 * TN), n_token_tiles, grid,
                                        (uint64_t)slice_entries * 16 * a.g.M_pad, (uint64_t)n * a.g.idx_row_bytes,
                                        a.g.tune_xcd_col_split);
+    snprintf(a.last_gather, sizeof(a.last_gather), "gather_onehot_kernel<%d, %d, %s, %d>", TN, TM, P8 ? "true" : "false", GS);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(OH_THREADS), LDS, ctx->stream, d_idx,
                        reinterpret_cast<const int8_t*>(a.d_lut), d_out, d_acc, n, a.g.M, slice_entries,
                        a.g.idx_row_bytes, n_token_tiles, n_items, ep, xmap);
@@ -1060,6 +1063,7 @@ int launch_i8(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_
     const uint32_t per_cu = LDS > 0 ? (uint32_t)(ctx->prop.maxSharedMemoryPerMultiProcessor / LDS) : 1;
     uint32_t grid = ctx->prop.multiProcessorCount * (per_cu < 1 ? 1 : per_cu > 2 ? 2 : per_cu);
     if (grid > n_items) grid = n_items;
+    snprintf(a.last_gather, sizeof(a.last_gather), "gather_i8_kernel<%d, %d, %d, %d, %d>", C_T, Q, GQ, TG, IDX_BITS);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(GATHER_THREADS), LDS, ctx->stream, d_idx,
                        reinterpret_cast<const int8_t*>(a.d_lut), d_out, d_acc, n, a.g.M, a.g.CB_pad,
                        a.g.idx_row_bytes, n_token_tiles, n_items, ep);
@@ -1083,6 +1087,7 @@ int launch_f32_impl(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, 
     const uint64_t wgs = (uint64_t)n_token_tiles * colblocks;
     if (wgs > 0x7FFFFFFFull) return set_error(ctx, PIMDL_ERR_UNSUPPORTED, "gather: %llu workgroups", (unsigned long long)wgs);
     const uint32_t by_xcd = colblocks % 8 == 0 ? 1u : 0u;
+    snprintf(a.last_gather, sizeof(a.last_gather), "gather_f32_kernel<%d, %d, %d, %d, %s, %d>", C_T, Q, GS, IDX_BITS, GROUPED ? "true" : "false", TPL);
     hipLaunchKernelGGL(kern, dim3((uint32_t)wgs), dim3(GF_THREADS), LDS, ctx->stream, d_idx,
                        reinterpret_cast<const float*>(a.d_lut), d_out, n, a.g.M, a.g.CB_pad, a.g.idx_row_bytes,
                        a.d_bias, a.d_scales, a.g.CB, a.desc.scale_group, a.desc.activation, n_token_tiles, by_xcd);

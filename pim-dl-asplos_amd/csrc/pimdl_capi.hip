@@ -927,6 +927,14 @@ int pimdl_get_device_info(pimdl_ctx* ctx, pimdl_device_info* info)
     return PIMDL_OK;
 }
 
+int pimdl_amm_last_gather_kernel(const pimdl_amm* a, char* name, size_t len)
+{
+    if (!a || !name || len == 0) return PIMDL_ERR_INVALID;
+    strncpy(name, a->last_gather, len - 1);
+    name[len - 1] = 0;
+    return PIMDL_OK;
+}
+
 int pimdl_amm_get_geometry(const pimdl_amm* a, pimdl_amm_geometry* out)
 {
     if (!a || !out) return PIMDL_ERR_INVALID;
