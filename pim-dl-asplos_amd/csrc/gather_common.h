@@ -118,6 +118,12 @@ __device__ __forceinline__ void lds_read32(uint32_t& dst, uint32_t addr)
     asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
 }
 
+template <int OFF>
+__device__ __forceinline__ void lds_read_u8(uint32_t& dst, uint32_t addr)
+{
+    asm volatile("ds_read_u8 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+
 // Loads through the scalar data cache (read only) of wave-uniform addresses; they count on the
 // scalar/LDS counter, not on the vector-memory counter.
 typedef float floatx16 __attribute__((ext_vector_type(16)));

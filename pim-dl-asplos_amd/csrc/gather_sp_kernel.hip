@@ -74,6 +74,15 @@ __device__ __forceinline__ void lgkm_wait()
     asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N < 15 ? N : 15) : "memory");
 }
 
+// a pointer that is the same in every lane, moved to scalar registers
+template <class T>
+__device__ __forceinline__ T* uniform_ptr(T* p)
+{
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<T*>(((uint64_t)hi << 32) | lo);
+}
+
 template <int TN, int TM, int GS>
 __global__ __launch_bounds__(SP_THREADS, 2) void gather_sparse_kernel(
     const uint8_t* __restrict__ idx, const int8_t* __restrict__ lut, float* __restrict__ out,
@@ -126,7 +135,6 @@ __global__ __launch_bounds__(SP_THREADS, 2) void gather_sparse_kernel(
     auto tok_tile_of = [&](uint32_t p) { uint32_t c, t; xmap.decode(p, n_token_tiles, c, t); return t; };
     uint32_t lut_item = blockIdx.x, lut_s = 0, ix_item = blockIdx.x, ix_s = 0;
     const int8_t* dma_base;   // uniform: start of the slice at the LUT stream position
-    const uint32_t dma_lane = wave * 1024 + lane * 16;
     const uint8_t* ix_base;   // uniform: the 256-byte block of index words at the index stream position
     uint32_t ix_lane_off;
     auto locate_lut = [&]() { dma_base = lut + (size_t)col_of(lut_item) * CB_pad * (WN * 16); };
@@ -138,16 +146,29 @@ __global__ __launch_bounds__(SP_THREADS, 2) void gather_sparse_kernel(
         ix_base = idx + (size_t)op * ep.op_idx_stride + (size_t)blk * idx_row_bytes * 64;
         ix_lane_off = lane * 4;
     };
-    // real = false (past the end of the stream): the operation re-copies the first slice of the table into a
+    // A wave copies DMA_PER_WAVE consecutive 1 KB blocks of a slice.  All of a slice's operations share one
+    // global address (the wave's part of the slice, per lane) and one LDS address; the block is chosen by the
+    // instruction's immediate offset, which the hardware adds to both.  The offset field reaches 4 KB, so blocks
+    // beyond the fourth go through a second address pair 4 KB further on.
+    // fetch = false (past the end of the stream): the operations re-copy the first slice of the table into a
     // buffer nobody reads any more, so that every slice issues the same number of operations and the waits
-    // can count them
-    auto lut_op = [&](uint32_t buf, bool real, auto uc) {
-        constexpr int u = decltype(uc)::value;
-        const uint32_t dst = BUF0 + buf * SLICE + wave * 1024;
-        const uint32_t off = (wave + SP_WAVES * u < NBLK) ? SP_WAVES * u * 1024 : 0;
-        const int8_t* src = (real ? dma_base : lut) + off;
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + dma_lane),
-                                         (__attribute__((address_space(3))) void*)(smem + dst + off), 16, 0, 0);
+    // can count them.
+    static_assert(NBLK % SP_WAVES == 0 && DMA_PER_WAVE <= 8, "whole blocks per wave, two address pairs");
+    const uint32_t dma_wave = wave * (DMA_PER_WAVE * 1024);
+    const uint32_t dma_lane = dma_wave + lane * 16;
+    const int8_t* lut_src = nullptr;  // this slice's source for this lane
+    uint32_t lut_dst = 0;             // ... and the wave's destination in LDS
+    // buf_off: byte offset of the destination buffer among the slice buffers
+    auto lut_begin = [&](uint32_t buf_off, bool fetch) {
+        // the choice is uniform: made once on the scalar side, not per lane
+        const int8_t* base = uniform_ptr(fetch ? dma_base : lut);
+        lut_src = base + dma_lane;
+        lut_dst = BUF0 + buf_off + dma_wave;
+    };
+    auto lut_op = [&](auto uc) {
+        constexpr int u = decltype(uc)::value, hi = u / 4, lo = u % 4;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(lut_src + hi * 4096),
+                                         (__attribute__((address_space(3))) void*)(smem + lut_dst + hi * 4096), 16, lo * 1024, 0);
     };
     auto lut_advance = [&]() {
         dma_base += SLICE;
@@ -158,15 +179,22 @@ __global__ __launch_bounds__(SP_THREADS, 2) void gather_sparse_kernel(
         }
     };
     auto stage_lut = [&](uint32_t buf) {
-        static_for<0, DMA_PER_WAVE>([&](auto uc) { lut_op(buf, true, uc); });
+        lut_begin(buf * SLICE, true);
+        static_for<0, DMA_PER_WAVE>([&](auto uc) { lut_op(uc); });
         lut_advance();
     };
-    auto ix_op = [&](uint32_t ibuf, bool real, auto ic) {
+    // index words: the same scheme, 256 bytes (64 tokens x one word) per operation
+    const uint8_t* ix_src = nullptr;
+    uint32_t ix_dst = 0;
+    auto ix_begin = [&](uint32_t ibuf_off, bool fetch) {
+        const uint8_t* base = uniform_ptr(fetch ? ix_base : idx);  // idx itself: any 64 tokens' words, never read
+        ix_src = base + ix_lane_off;
+        ix_dst = IBUF0 + ibuf_off + wave * IWAVE;
+    };
+    auto ix_op = [&](auto ic) {
         constexpr int i = decltype(ic)::value;
-        const uint32_t dst = IBUF0 + ibuf * IBYTES + wave * IWAVE;
-        const uint8_t* src = real ? ix_base + 256 * i : idx;
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + (real ? ix_lane_off : 0u)),
-                                         (__attribute__((address_space(3))) void*)(smem + dst + 256 * i), 4, 0, 0);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)ix_src,
+                                         (__attribute__((address_space(3))) void*)(smem + ix_dst), 4, 256 * i, 0);
     };
     auto ix_advance = [&]() {
         ix_base += IWORDS * 256;
@@ -177,18 +205,19 @@ __global__ __launch_bounds__(SP_THREADS, 2) void gather_sparse_kernel(
         }
     };
     auto stage_ix = [&](uint32_t ibuf) {
-        static_for<0, IX_OPS>([&](auto ic) { ix_op(ibuf, true, ic); });
+        ix_begin(ibuf * IBYTES, true);
+        static_for<0, IX_OPS>([&](auto ic) { ix_op(ic); });
         ix_advance();
     };
-    // Index word k of a token holds the nibbles of codebooks 8k .. 8k+7 of the slice; this lane's two are byte g.
-    // Stored pre-masked twice, so that one v_bfe_u32 yields nibble * 16, the table entry's offset.
-    const uint32_t byte_shift = 8 * g;
-    const uint32_t ix_lane = IBUF0 + wave * IWAVE + (((wave * (TM * 16)) & 63) + j) * 4;
-    auto read_ix = [&](uint32_t (&raw)[TM][IWORDS], uint32_t ibuf) {
-        const uint32_t addr = ix_lane + ibuf * IBYTES;
+    // Index word k of a token holds the nibbles of codebooks 8k .. 8k+7 of the slice; this lane's two are byte g,
+    // which it reads on its own (the four lane groups read the four bytes of the same word: one bank, broadcast).
+    // Kept as the two table offsets, nibble * 16.
+    const uint32_t ix_lane = IBUF0 + wave * IWAVE + (((wave * (TM * 16)) & 63) + j) * 4 + g;
+    auto read_ix = [&](uint32_t (&raw)[TM][IWORDS], uint32_t ibuf_off) {
+        const uint32_t addr = ix_lane + ibuf_off;
         static_for<0, TM * IWORDS>([&](auto ec) {
             constexpr int t = decltype(ec)::value / IWORDS, i = decltype(ec)::value % IWORDS;
-            lds_read32<(i * 64 + t * 16) * 4>(raw[t][i], addr);
+            lds_read_u8<(i * 64 + t * 16) * 4>(raw[t][i], addr);
         });
     };
     auto unpack_ix = [&](uint32_t (&lo)[TM][IWORDS], uint32_t (&hi)[TM][IWORDS], uint32_t (&raw)[TM][IWORDS]) {
@@ -201,8 +230,8 @@ __global__ __launch_bounds__(SP_THREADS, 2) void gather_sparse_kernel(
         for (int t = 0; t < TM; ++t)
 #pragma unroll
             for (int i = 0; i < IWORDS; ++i) {
-                lo[t][i] = (raw[t][i] << 4) & 0xF0F0F0F0u;
-                hi[t][i] = raw[t][i] & 0xF0F0F0F0u;
+                lo[t][i] = (raw[t][i] << 4) & 0xF0u;
+                hi[t][i] = raw[t][i] & 0xF0u;
             }
     };
 
@@ -301,7 +330,9 @@ __global__ __launch_bounds__(SP_THREADS, 2) void gather_sparse_kernel(
 
     uint32_t item0 = blockIdx.x;
     const uint32_t b_lane = BUF0 + (g * WN + j) * 16;  // this lane's 16 bytes of codebook g, column position j
-    uint32_t buf = 0, ibuf_next = 1;
+    // byte offsets of the buffers in their rings: the slice being read and the one its copies go into (the
+    // slice before), the index words read next and the ones copied into
+    uint32_t cur_off = 0, copy_off = (NBUF - 1) * SLICE, ixn_off = IBYTES, ixc_off = 0;
     uint32_t k = 0;
     bool stores_behind = false;
     constexpr bool COUNT_STORES = (PD - 1) * DMA_OPS + EPI_STORES <= 63;  // memory counter range
@@ -319,9 +350,9 @@ __global__ __launch_bounds__(SP_THREADS, 2) void gather_sparse_kernel(
         }
         const bool fetch = k + PD < total;
         const bool fetch_ix = k + PD + 1 < total;
-        const uint32_t lbp = buf >= 1 ? buf - 1 : NBUF - 1;
-        const uint32_t ibp = ibuf_next >= 1 ? ibuf_next - 1 : NIBUF - 1;
-        const uint32_t bbase = buf * SLICE + b_lane;
+        const uint32_t bbase = cur_off + b_lane;
+        lut_begin(copy_off, fetch);
+        ix_begin(ixc_off, fetch_ix);
 
         // Operand registers: the dense operand of a column group is re-armed with the next K-step's bytes as
         // soon as its TM instructions have been issued; the sparse operand is double buffered.
@@ -337,8 +368,7 @@ __global__ __launch_bounds__(SP_THREADS, 2) void gather_sparse_kernel(
             constexpr int ks = decltype(ksc)::value;
 #pragma unroll
             for (int t = 0; t < TM; ++t) {
-                const uint32_t e0 = __builtin_amdgcn_ubfe(iw_lo[t][ks], byte_shift, 8);
-                const uint32_t e1 = __builtin_amdgcn_ubfe(iw_hi[t][ks], byte_shift, 8);
+                const uint32_t e0 = iw_lo[t][ks], e1 = iw_hi[t][ks];
                 lds_read64<0>(a_lo[ks & 1][t], e0);
                 lds_read32<8>(p_lo[ks & 1][t], e0);
                 lds_read64<0>(a_hi[ks & 1][t], e1);
@@ -378,15 +408,15 @@ __global__ __launch_bounds__(SP_THREADS, 2) void gather_sparse_kernel(
                     issue_b(std::integral_constant<int, ks + 1>{}, cc);
                     if constexpr (c == 0) issue_a(std::integral_constant<int, ks + 1>{});
                 } else if constexpr (c == 0) {
-                    read_ix(iw_raw, ibuf_next);  // the next slice's index words (this wave's own copy, landed)
+                    read_ix(iw_raw, ixn_off);  // the next slice's index words (this wave's own copy, landed)
                 }
                 // this slice's copy operations (slice k+PD of the table, index words k+PD+1), a few per column group
                 constexpr int IK = PD == 1 ? KSTEPS * TN / 2 : KSTEPS * TN;
                 constexpr int pos = ks * TN + c;
                 static_for<(pos < IK ? pos : IK) * DMA_OPS / IK, (pos + 1 < IK ? pos + 1 : IK) * DMA_OPS / IK>([&](auto oc) {
                     constexpr int o = decltype(oc)::value;
-                    if constexpr (o < DMA_PER_WAVE) lut_op(lbp, fetch, std::integral_constant<int, o>{});
-                    else ix_op(ibp, fetch_ix, std::integral_constant<int, o - DMA_PER_WAVE>{});
+                    if constexpr (o < DMA_PER_WAVE) lut_op(std::integral_constant<int, o>{});
+                    else ix_op(std::integral_constant<int, o - DMA_PER_WAVE>{});
                 });
                 __builtin_amdgcn_sched_barrier(0);
             });
@@ -397,8 +427,10 @@ __global__ __launch_bounds__(SP_THREADS, 2) void gather_sparse_kernel(
         }
         unpack_ix(iw_lo, iw_hi, iw_raw);
 
-        buf = buf + 1 == NBUF ? 0 : buf + 1;
-        ibuf_next = ibuf_next + 1 == NIBUF ? 0 : ibuf_next + 1;
+        copy_off = cur_off;
+        cur_off = cur_off + SLICE == NBUF * SLICE ? 0 : cur_off + SLICE;
+        ixc_off = ixn_off;
+        ixn_off = ixn_off + IBYTES == NIBUF * IBYTES ? 0 : ixn_off + IBYTES;
     }
     stores_behind = epilogue(item0);
     }
