@@ -358,7 +358,7 @@ __global__ __launch_bounds__(SP_THREADS, 2) void gather_sparse_kernel(
         // soon as its TM instructions have been issued; the sparse operand is double buffered.
         v4i b_lo[TN], b_hi[TN];
         v2i a_lo[2][TM], a_hi[2][TM];
-        uint32_t p_lo[2][TM], p_hi[2][TM];
+        v2i p_lo[2][TM], p_hi[2][TM];  // both position words of an entry: 8-byte reads of the table do not meet in a bank, 4-byte reads do
         auto issue_b = [&](auto ksc, auto cc) {
             constexpr int ks = decltype(ksc)::value, c = decltype(cc)::value;
             lds_read<((8 * ks) * WN + c * 16) * 16>(b_lo[c], bbase);
@@ -370,9 +370,9 @@ __global__ __launch_bounds__(SP_THREADS, 2) void gather_sparse_kernel(
             for (int t = 0; t < TM; ++t) {
                 const uint32_t e0 = iw_lo[t][ks], e1 = iw_hi[t][ks];
                 lds_read64<0>(a_lo[ks & 1][t], e0);
-                lds_read32<8>(p_lo[ks & 1][t], e0);
+                lds_read64<8>(p_lo[ks & 1][t], e0);
                 lds_read64<0>(a_hi[ks & 1][t], e1);
-                lds_read32<12>(p_hi[ks & 1][t], e1);
+                lds_read64<8>(p_hi[ks & 1][t], e1);
             }
         };
         // slice prologue: sparse operand first, then the dense operand of every column group, in this order
@@ -401,7 +401,7 @@ __global__ __launch_bounds__(SP_THREADS, 2) void gather_sparse_kernel(
 #pragma unroll
                 for (int t = 0; t < TM; ++t) {
                     const v4i aa = {a_lo[ks & 1][t][0], a_lo[ks & 1][t][1], a_hi[ks & 1][t][0], a_hi[ks & 1][t][1]};
-                    acc[t][c] = __builtin_amdgcn_smfmac_i32_16x16x128_i8(aa, bb, acc[t][c], (int)(p_lo[ks & 1][t] | p_hi[ks & 1][t]), 0, 0);
+                    acc[t][c] = __builtin_amdgcn_smfmac_i32_16x16x128_i8(aa, bb, acc[t][c], (int)(p_lo[ks & 1][t][0] | p_hi[ks & 1][t][1]), 0, 0);
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 if constexpr (!LAST) {
