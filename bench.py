@@ -133,6 +133,14 @@ def cpu_baseline(shapes, N, warmup=10, rounds=20, budget_s=25.0):
                       f"flags (-O3 -fopenmp, no -march), {threads} OpenMP threads, {dt * 1e3:.1f} ms per round"}
 
 
+def settled_profile(amm, x, N, y, iters):
+    """pimdl_amm_profile after enough warm-up launches (about 30 ms of them) for the engine clock to have ramped
+    up again: preparing an operator on the host leaves the GPU idle for a second, and the clock drops meanwhile."""
+    t = amm.profile(x.data_ptr(), N, y.data_ptr(), warmup=2, iters=2)
+    warm = int(min(2000, max(5, 30.0 / max(t["total_ms"], 1e-3))))
+    return amm.profile(x.data_ptr(), N, y.data_ptr(), warmup=warm, iters=iters)
+
+
 def per_codebook_scale(pimdl, ctx, rng, N, shapes, iters=20):
     """The same pair with one fp32 scale per codebook (scale_group = 1), the wording of the benchmark
     configuration; the reference itself has one scale per tensor, which is what `value` measures.  A different
@@ -148,7 +156,7 @@ def per_codebook_scale(pimdl, ctx, rng, N, shapes, iters=20):
         amm = ctx.amm(cent, lut, scales, None, max_n=N, scale_group=1)
         x = torch.randn((N, K), device="cuda", dtype=torch.float32)
         y = torch.empty((N, M), device="cuda", dtype=torch.float32)
-        t = amm.profile(x.data_ptr(), N, y.data_ptr(), warmup=20, iters=iters)
+        t = settled_profile(amm, x, N, y, iters)
         out.append({"K": K, "M": M, "ccs_ms": t["ccs_ms"], "gather_ms": t["gather_ms"], "amm_ms": t["total_ms"],
                     "gather_kernel": amm.last_gather_kernel()})
         amm.close()
@@ -178,7 +186,7 @@ def vit_sweep(pimdl, ctx, iters=10):
                     else:
                         lut, scales = rng.standard_normal((CB, C, M), dtype=np.float32), None
                     amm = ctx.amm(cent, lut, scales, None, max_n=N)
-                    t = amm.profile(x.data_ptr(), N, y.data_ptr(), warmup=5, iters=iters)
+                    t = settled_profile(amm, x, N, y, iters)
                     e = 1 if kind == "i8" else 4
                     cells.append({"K": K, "M": M, "v": v, "C": C, "lut": kind, "ccs_us": round(t["ccs_ms"] * 1e3, 1),
                                   "gather_us": round(t["gather_ms"] * 1e3, 1),
