@@ -499,9 +499,10 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
     // the explicit ones.  Two independent stream positions step through the (item, slice) sequence:
     // the LUT position runs PD slices ahead of the one being consumed, the index position PD+1
     // (the index words of slice k+1 are unpacked while slice k is multiplied).
-    //   LUT:   wave w copies the 1 KB blocks w, w+8, .. of a slice; where the blocks do not divide
-    //          evenly a wave copies its first block twice, so that every wave issues the same
-    //          number of operations per slice (the waits below count them).
+    //   LUT:   wave w copies DMA_PER_WAVE consecutive 1 KB blocks of a slice.  All of a slice's operations
+    //          share one global address (per lane) and one LDS address; the block is chosen by the
+    //          instruction's immediate offset, which the hardware adds to both (the field reaches 4 KB, so
+    //          blocks beyond the fourth go through a second address pair 4 KB further on).
     //   index: lane L of wave w copies index word i of token 64 w + L with its i-th operation,
     //          into [wave][word][64 tokens]; only the wave itself reads them back.
     // Addresses are kept as a wave-uniform 64-bit base (scalar registers) plus a 32-bit per-lane
@@ -509,8 +510,10 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
     auto col_of = [&](uint32_t p) { uint32_t c, t; xmap.decode(p, n_token_tiles, c, t); return c; };
     auto tok_tile_of = [&](uint32_t p) { uint32_t c, t; xmap.decode(p, n_token_tiles, c, t); return t; };
     uint32_t lut_item = blockIdx.x, lut_s = 0, ix_item = blockIdx.x, ix_s = 0;
+    static_assert(NBLK % OH_WAVES == 0 && DMA_PER_WAVE <= 8, "whole blocks per wave, two address pairs");
     const int8_t* dma_base;   // uniform: start of the slice at the LUT stream position
-    const uint32_t dma_lane = wave * 1024 + lane * 16;
+    const uint32_t dma_wave = wave * (DMA_PER_WAVE * 1024);
+    const uint32_t dma_lane = dma_wave + lane * 16;
     const uint8_t* ix_base;   // uniform: the 256-byte block of index words at the index stream position
     uint32_t ix_lane_off;     // per lane: its token's word inside a block
     auto locate_lut = [&]() {
@@ -527,16 +530,19 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
         ix_base = idx + (size_t)op * ep.op_idx_stride + (size_t)blk * idx_row_bytes * 64;
         ix_lane_off = lane * 4;
     };
-    // real = false (past the end of the stream): the operation re-copies the first slice of the
+    // fetch = false (past the end of the stream): the operations re-copy the first slice of the
     // LUT into a buffer nobody reads any more, so that every slice issues the same number of
     // operations and the waits can count them
-    auto lut_op = [&](uint32_t buf, bool real, auto uc) {
-        constexpr int u = decltype(uc)::value;
-        const uint32_t dst = BUF0 + buf * SLICE + wave * 1024;  // wave-uniform; lanes add 16*lane
-        const uint32_t off = (wave + OH_WAVES * u < NBLK) ? OH_WAVES * u * 1024 : 0;  // wave-uniform
-        const int8_t* src = (real ? dma_base : lut) + off;  // uniform
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + dma_lane),
-                                         (__attribute__((address_space(3))) void*)(smem + dst + off), 16, 0, 0);
+    const int8_t* lut_src = nullptr;  // this slice's source for this lane
+    uint32_t lut_dst = 0;             // ... and the wave's destination in LDS
+    auto lut_begin = [&](uint32_t buf, bool fetch) {
+        lut_src = (fetch ? dma_base : lut) + dma_lane;
+        lut_dst = BUF0 + buf * SLICE + dma_wave;
+    };
+    auto lut_op = [&](auto uc) {
+        constexpr int u = decltype(uc)::value, hi = u / 4, lo = u % 4;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(lut_src + hi * 4096),
+                                         (__attribute__((address_space(3))) void*)(smem + lut_dst + hi * 4096), 16, lo * 1024, 0);
     };
     auto lut_advance = [&]() {
         dma_base += SLICE;
@@ -547,16 +553,22 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
         }
     };
     auto stage_lut = [&](uint32_t buf) {
-        static_for<0, DMA_PER_WAVE>([&](auto uc) { lut_op(buf, true, uc); });
+        lut_begin(buf, true);
+        static_for<0, DMA_PER_WAVE>([&](auto uc) { lut_op(uc); });
         lut_advance();
     };
-    // real = false: as above, into an index buffer nobody will unpack
-    auto ix_op = [&](uint32_t ibuf, bool real, auto ic) {
+    // index words: the same scheme, 256 bytes (64 tokens x one word) per operation; fetch = false: as above,
+    // into an index buffer nobody will unpack (from the start of the index buffer: any 64 tokens' words)
+    const uint8_t* ix_src = nullptr;
+    uint32_t ix_dst = 0;
+    auto ix_begin = [&](uint32_t ibuf, bool fetch) {
+        ix_src = (fetch ? ix_base : idx) + ix_lane_off;
+        ix_dst = IBUF0 + ibuf * IBYTES + wave * IWAVE;
+    };
+    auto ix_op = [&](auto ic) {
         constexpr int i = decltype(ic)::value;
-        const uint32_t dst = IBUF0 + ibuf * IBYTES + wave * IWAVE;  // wave-uniform; lanes add 4*lane
-        const uint8_t* src = real ? ix_base + 256 * i : idx;  // uniform
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + (real ? ix_lane_off : 0u)),
-                                         (__attribute__((address_space(3))) void*)(smem + dst + 256 * i), 4, 0, 0);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)ix_src,
+                                         (__attribute__((address_space(3))) void*)(smem + ix_dst), 4, 256 * i, 0);
     };
     auto ix_advance = [&]() {
         ix_base += IWORDS * 256;
@@ -567,7 +579,8 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
         }
     };
     auto stage_ix = [&](uint32_t ibuf) {
-        static_for<0, IX_OPS>([&](auto ic) { ix_op(ibuf, true, ic); });
+        ix_begin(ibuf, true);
+        static_for<0, IX_OPS>([&](auto ic) { ix_op(ic); });
         ix_advance();
     };
     // This lane's nibble of K-step ks is nibble 4 (ks & 1) + g of index word ks / 2.  Shifting the
@@ -733,6 +746,8 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
         const uint32_t lbp = buf >= 1 ? buf - 1 : NBUF - 1;               // (k + PD) % NBUF = (k - 1) % NBUF
         const uint32_t ibp = ibuf_next >= 1 ? ibuf_next - 1 : NIBUF - 1;  // (k + PD + 1) % NIBUF = k % NIBUF
         const uint32_t abase = buf * SLICE + a_lane;
+        lut_begin(lbp, fetch);
+        ix_begin(ibp, fetch_ix);
 
         v4i a_op[2][TN], b_op[2][TM];
         // K-step ks covers codebooks 4 ks .. 4 ks + 3 of the slice; this lane's is 4 ks + g.
@@ -763,8 +778,8 @@ __global__ __launch_bounds__(OH_THREADS, 2) void gather_onehot_kernel(
             constexpr int IK = PD == 1 ? KSTEPS / 2 : KSTEPS;
             static_for<(ks < IK ? ks : IK) * DMA_OPS / IK, (ks + 1 < IK ? ks + 1 : IK) * DMA_OPS / IK>([&](auto oc) {
                 constexpr int o = decltype(oc)::value;
-                if constexpr (o < DMA_PER_WAVE) lut_op(lbp, fetch, std::integral_constant<int, o>{});
-                else ix_op(ibp, fetch_ix, std::integral_constant<int, o - DMA_PER_WAVE>{});
+                if constexpr (o < DMA_PER_WAVE) lut_op(std::integral_constant<int, o>{});
+                else ix_op(std::integral_constant<int, o - DMA_PER_WAVE>{});
             });
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
