@@ -79,6 +79,26 @@ def test_vit_base_ffn2_sweep_full_batch(env, v, C, lut_kind):
     run_and_check_sample(env[1], 29 + v + C, 12608, 3072, v, C, 768, lut_kind, sample=64)
 
 
+# The shapes of the reference's sensitivity-analysis configurations (asplos24-ae/sensitivity-analysis/configs):
+#   hidden-dim/dim{1024,2048,2560,4096,5120}.yaml   token_dim d, ffn 4d, 256 codebooks for QKV/O/FFN1 and 1024 for
+#                                                   FFN2, i.e. sub_vec_len d/256 = 4, 8, 10, 16, 20; 16 centroids
+#   bert-base/sub-vector-length/v{2,4,8,16,32}.yaml QKV codebooks 384, 192, 96, 48, 24
+#   bert-base/centroid-number/ct{8,16,32,64,128}.yaml
+#   vit-huge/*                                      token_dim 1280 (320 codebooks), ffn 5120 (1280 codebooks)
+# Rows are independent, so the batch is cut from the configurations' 64 x 512 tokens to 2048 (ViT-huge: 8 x 264).
+ENVELOPE = (
+    [(f"hidden{d}-qkv", 2048, d, d // 256, 16, 3 * d) for d in (1024, 2048, 2560, 4096, 5120)] +
+    [(f"hidden{d}-ffn2", 2048, 4 * d, d // 256, 16, d) for d in (1024, 2048, 2560, 4096, 5120)] +
+    [(f"bert-base-v{v}-qkv", 2048, 768, v, 16, 2304) for v in (2, 4, 8, 16, 32)] +
+    [(f"bert-base-ct{c}-ffn2", 2048, 3072, 4, c, 768) for c in (8, 16, 32, 64, 128)] +
+    [("vit-huge-ffn1", 2112, 1280, 4, 16, 5120), ("vit-huge-ffn2", 2112, 5120, 4, 16, 1280)])
+
+
+@pytest.mark.parametrize("name,N,K,v,C,M", ENVELOPE, ids=[e[0] for e in ENVELOPE])
+def test_reference_sensitivity_analysis_shapes(env, name, N, K, v, C, M):
+    run_and_check_sample(env[1], 57 + K + v + C, N, K, v, C, M, "i8", sample=48)
+
+
 def test_reference_single_amm_search_space_shape(env):
     """The shape of the reference's 89 single-AMM tuning configs: N = 32768, 1024 -> 4096, 256 codebooks of
     16 centroids (512 MB of fp32 output, 128 token tiles x 64 column tiles)."""
