@@ -54,7 +54,9 @@ namespace {
 
 template <int V>
 struct CcsShape {
-    static constexpr int ROW_FLOATS = (2 * V > 32) ? 2 * V : 32;  // floats of one token per tile
+    // floats of one token per wave: 32, or 2 v above that, or 40 where v does not divide 32 (v = 10, 20)
+    static constexpr int ROW_FLOATS = (32 % V != 0) ? 40 : (2 * V > 32) ? 2 * V : 32;
+    static_assert(ROW_FLOATS % V == 0 && ROW_FLOATS % 4 == 0, "whole codebooks and whole 16-byte pieces per wave");
     static constexpr int CBT = ROW_FLOATS / V;                    // codebooks per workgroup
     static constexpr int WAVES = 4;                               // each wave: its own codebook group
     static constexpr int TILE_TOKENS = 64;                        // one token per lane
@@ -166,16 +168,25 @@ __global__ __launch_bounds__(CCS_THREADS) void ccs_kernel(const float* __restric
     // A tile is 64 tokens x 4*RF floats: rows of 4*RF*4 bytes (512 B for v <= 16) are contiguous in
     // HBM, and wave w searches the w-th quarter of the columns for all 64 tokens.
     constexpr int F4_PER_ROW = S::WAVES * RF / 4;
+    constexpr int PASSES = TT * F4_PER_ROW / CCS_THREADS;     // float4 per lane per tile (= RF / 4)
+    static_assert(TT * F4_PER_ROW % CCS_THREADS == 0, "the tile's 16-byte pieces divide among the threads");
+    // Piece e = threadIdx.x + CCS_THREADS * i of the tile is column piece e % F4_PER_ROW of row e / F4_PER_ROW.
+    // Where the threads cover whole rows per pass (256 % F4_PER_ROW == 0) that is the same column piece and
+    // a fixed row step in every pass; otherwise (40 pieces per row) both are worked out per pass.
+    constexpr bool WHOLE_ROWS = CCS_THREADS % F4_PER_ROW == 0;
     constexpr int ROWS_PER_PASS = CCS_THREADS / F4_PER_ROW;
-    constexpr int PASSES = TT / ROWS_PER_PASS;                // float4 per lane per tile (= RF / 4)
-    const uint32_t fq = threadIdx.x % F4_PER_ROW;
-    const uint32_t fr0 = threadIdx.x / F4_PER_ROW;
+    auto piece_row = [&](int i) -> uint32_t {
+        return WHOLE_ROWS ? threadIdx.x / F4_PER_ROW + i * ROWS_PER_PASS : (threadIdx.x + CCS_THREADS * i) / F4_PER_ROW;
+    };
+    auto piece_col = [&](int i) -> uint32_t {
+        return WHOLE_ROWS ? threadIdx.x % F4_PER_ROW : (threadIdx.x + CCS_THREADS * i) % F4_PER_ROW;
+    };
     auto fetch = [&](float4 (&pf)[PASSES], uint32_t tile_id) {
         const uint32_t t_tok0 = (tile_id / tiles_cb) * TT;
-        const uint32_t col = (tile_id % tiles_cb) * (S::WAVES * RF) + 4 * fq;
 #pragma unroll
         for (int i = 0; i < PASSES; ++i) {
-            uint32_t tok = t_tok0 + fr0 + i * ROWS_PER_PASS;
+            const uint32_t col = (tile_id % tiles_cb) * (S::WAVES * RF) + 4 * piece_col(i);
+            uint32_t tok = t_tok0 + piece_row(i);
             if (tok >= N) tok = N - 1;  // rows past N repeat the last token; never stored
             const float* src = x + (size_t)tok * K + col;
             if (vec_ok && col + 4 <= K) {
@@ -198,7 +209,7 @@ __global__ __launch_bounds__(CCS_THREADS) void ccs_kernel(const float* __restric
     // transpose through LDS: coalesced rows in, one row slice per lane out
 #pragma unroll
     for (int i = 0; i < PASSES; ++i)
-        *reinterpret_cast<float4*>(&tile[(fr0 + i * ROWS_PER_PASS) * PITCH + 4 * fq]) = pf[i];
+        *reinterpret_cast<float4*>(&tile[piece_row(i) * PITCH + 4 * piece_col(i)]) = pf[i];
     __syncthreads();
     float xv[RF];
 #pragma unroll
@@ -1248,7 +1259,9 @@ int launch_ccs_bits(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d
         case 2: return launch_ccs_t<2, IDX_BITS>(ctx, g, d_x, d_cent, d_idx, n);
         case 4: return launch_ccs_t<4, IDX_BITS>(ctx, g, d_x, d_cent, d_idx, n);
         case 8: return launch_ccs_t<8, IDX_BITS>(ctx, g, d_x, d_cent, d_idx, n);
+        case 10: return launch_ccs_t<10, IDX_BITS>(ctx, g, d_x, d_cent, d_idx, n);  // the reference's hidden-dim sweep:
         case 16: return launch_ccs_t<16, IDX_BITS>(ctx, g, d_x, d_cent, d_idx, n);
+        case 20: return launch_ccs_t<20, IDX_BITS>(ctx, g, d_x, d_cent, d_idx, n);  // token_dim 2560 and 5120 over 256 codebooks
         case 32: return launch_ccs_t<32, IDX_BITS>(ctx, g, d_x, d_cent, d_idx, n);
         default: {
             const uint64_t total = (uint64_t)n * (g.CB_pad / (8 / IDX_BITS));
@@ -1434,7 +1447,9 @@ uint32_t ccs_cb_per_wg(uint32_t v)
         case 2: return CcsShape<2>::WAVES * CcsShape<2>::CBT;
         case 4: return CcsShape<4>::WAVES * CcsShape<4>::CBT;
         case 8: return CcsShape<8>::WAVES * CcsShape<8>::CBT;
+        case 10: return CcsShape<10>::WAVES * CcsShape<10>::CBT;
         case 16: return CcsShape<16>::WAVES * CcsShape<16>::CBT;
+        case 20: return CcsShape<20>::WAVES * CcsShape<20>::CBT;
         case 32: return CcsShape<32>::WAVES * CcsShape<32>::CBT;
         default: return 0;
     }

@@ -93,6 +93,11 @@ def test_sweep_sub_vector_length_and_centroids(ctx, v, C):
     (300, 44, 4, 20, 40),    # 17..32 centroids on the matrix-core search: ids past C never win
     (129, 18, 2, 17, 24),    # same, v=2, CB=9
     (200, 72, 8, 31, 50),    # same, v=8
+    (333, 70, 10, 16, 52),   # sub_vec_len 10 (the reference's token_dim 2560 over 256 codebooks): CB=7, K % 4 != 0
+    (130, 170, 10, 12, 37),  # ... CB=17 (two codebook tiles, the second ragged), C not a power of two
+    (65, 640, 10, 40, 24),   # ... 8-bit indices, several centroid groups per codebook
+    (257, 60, 20, 16, 20),   # sub_vec_len 20 (token_dim 5120): CB=3
+    (100, 500, 20, 130, 16), # ... CB=25, more than 128 centroids
 ])
 def test_ragged_shapes(ctx, N, K, v, C, M):
     check_i8(ctx, N + K + M, N, K, v, C, M)
