@@ -65,11 +65,20 @@ def tune(ctx, pimdl, n, K, v, C, M, lut_dtype="int8", seed=0, iters=20, full=Tru
     x = torch.randn((n, K), device="cuda", dtype=torch.float32)
     y = torch.empty((n, M), device="cuda", dtype=torch.float32)
 
+    heated = [False]
+
     def timed(amm):
+        # the first measurement follows host work (table generation, upload) during which the GPU idled and its
+        # clock dropped: heat it up again with about 30 ms of the same launches before timing anything
+        if not heated[0]:
+            t = amm.profile(x.data_ptr(), n, y.data_ptr(), warmup=2, iters=2)
+            amm.profile(x.data_ptr(), n, y.data_ptr(), warmup=int(min(2000, max(5, 30.0 / max(t["total_ms"], 1e-3)))), iters=1)
+            heated[0] = True
         t = amm.profile(x.data_ptr(), n, y.data_ptr(), warmup=3, iters=iters)
         return t["ccs_ms"], t["gather_ms"]
 
     def build(**fields):
+        heated[0] = False
         try:
             return ctx.amm(cent, lut, scales, None, max_n=n, tuning=fields)
         except pimdl.PimdlError as e:
