@@ -149,9 +149,11 @@ typedef enum pimdl_search_kernel {
 typedef struct pimdl_amm_tuning {
     uint32_t col_block;      /* output columns per work item of the gather: 48, 64 or 96 (what the kernel offers) */
     uint32_t gather_kernel;  /* pimdl_gather_kernel; fixes the layout of the resident table */
-    uint32_t token_item;     /* tokens per work item of the matrix-core gathers: 128 or 256 */
+    uint32_t token_item;     /* tokens per work item of the matrix-core gathers: 128 or 256; the sparse kernel
+                                also 512 (one workgroup of eight waves per CU instead of two of four) */
     uint32_t cb_per_slice;   /* codebooks staged in LDS at a time by the matrix-core gathers: 16 or 32
-                                (32 needs col_block <= 64 and num_codebook padded to a multiple of 32) */
+                                (32 needs col_block <= 64, or 512-token items); 64 with 512-token items and
+                                col_block 48, num_codebook padded to a multiple of 64 */
     uint32_t xcd_col_split;  /* how the 8 XCDs (each with its own L2) share the work items of the matrix-core
                                 gathers: 1, 2, 4 or 8 of them along the column tiles, the rest along the token
                                 tiles; PIMDL_XCD_PLAIN = no dealing.  A split that does not divide a launch's
@@ -337,7 +339,10 @@ typedef struct pimdl_device_info {
     uint64_t hbm_bytes;
 } pimdl_device_info;
 PIMDL_API int pimdl_get_device_info(pimdl_ctx* ctx, pimdl_device_info* info);
-/* Geometry the operator's kernels were launched with (for documentation of a measurement). */
+/* Geometry of the operator's kernels (for documentation of a measurement).  The gather launcher picks the slice
+ * depth, the tokens per workgroup and with them the LDS bytes and threads by the batch it is given:
+ * cb_per_slice, lds_bytes, tokens_per_wg and gather_threads are those of the last launch, or the plan's defaults
+ * before the first. */
 typedef struct pimdl_amm_geometry {
     uint32_t num_codebook, num_codebook_padded, idx_bits, idx_row_bytes;
     uint32_t col_block, row_pitch, cb_per_slice, lds_bytes, tokens_per_wg, gather_threads;

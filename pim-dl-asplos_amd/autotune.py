@@ -8,8 +8,8 @@ would otherwise decide by rule (pimdl_amm_tuning):
 
     gather_kernel   how entries are accumulated: byte adder / dense one-hot / sparse one-hot matrix kernel
     col_block       output columns per work item (48, 64, 96)
-    token_item      tokens per work item (128, 256)
-    cb_per_slice    codebooks staged in LDS at a time (16, 32)
+    token_item      tokens per work item (128, 256; 512 = eight waves per workgroup, sparse kernel)
+    cb_per_slice    codebooks staged in LDS at a time (16, 32, 64)
     xcd_col_split   how the 8 XCDs share column tiles and token tiles (1, 2, 4, 8, plain order)
     search_kernel   closest-centroid search: lane-per-token scan / fp32 matrix core / bf16 matrix core
     search_token_tile  tokens per tile of the bf16 search (64, 128)
@@ -36,7 +36,7 @@ COL_BLOCKS = (48, 64, 96)
 GATHER_KERNELS = {"rows": 1, "onehot": 2, "sparse": 3}
 SEARCH_KERNELS = {"scan": 1, "mfma_f32": 2, "mfma_bf16": 3}
 XCD_PLAIN = 0xFFFFFFFF
-RUNTIME_GATHER = {"token_item": (128, 256), "cb_per_slice": (16, 32), "xcd_col_split": (1, 2, 4, 8, XCD_PLAIN)}
+RUNTIME_GATHER = {"token_item": (128, 256, 512), "cb_per_slice": (16, 32, 64), "xcd_col_split": (1, 2, 4, 8, XCD_PLAIN)}
 
 
 def shape_key(device, n, K, v, C, M, dtype):

@@ -827,6 +827,7 @@ int launch_onehot_tm(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out,
                                        (uint64_t)slice_entries * 16 * a.g.M_pad, (uint64_t)n * a.g.idx_row_bytes,
                                        a.g.tune_xcd_col_split);
     snprintf(a.last_gather, sizeof(a.last_gather), "gather_onehot_kernel<%d, %d, %s, %d>", TN, TM, P8 ? "true" : "false", GS);
+    a.note_launch(GS, LDS, OH_TOK_ITEM, OH_THREADS);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(OH_THREADS), LDS, ctx->stream, d_idx,
                        reinterpret_cast<const int8_t*>(a.d_lut), d_out, d_acc, n, a.g.M, slice_entries,
                        a.g.idx_row_bytes, n_token_tiles, n_items, ep, xmap);
@@ -1079,6 +1080,7 @@ int launch_i8(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_
     uint32_t grid = ctx->prop.multiProcessorCount * (per_cu < 1 ? 1 : per_cu > 2 ? 2 : per_cu);
     if (grid > n_items) grid = n_items;
     snprintf(a.last_gather, sizeof(a.last_gather), "gather_i8_kernel<%d, %d, %d, %d, %d>", C_T, Q, GQ, TG, IDX_BITS);
+    a.note_launch(4 * GQ, LDS, TOK_ITEM, GATHER_THREADS);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(GATHER_THREADS), LDS, ctx->stream, d_idx,
                        reinterpret_cast<const int8_t*>(a.d_lut), d_out, d_acc, n, a.g.M, a.g.CB_pad,
                        a.g.idx_row_bytes, n_token_tiles, n_items, ep);
@@ -1103,6 +1105,7 @@ int launch_f32_impl(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, 
     if (wgs > 0x7FFFFFFFull) return set_error(ctx, PIMDL_ERR_UNSUPPORTED, "gather: %llu workgroups", (unsigned long long)wgs);
     const uint32_t by_xcd = colblocks % 8 == 0 ? 1u : 0u;
     snprintf(a.last_gather, sizeof(a.last_gather), "gather_f32_kernel<%d, %d, %d, %d, %s, %d>", C_T, Q, GS, IDX_BITS, GROUPED ? "true" : "false", TPL);
+    a.note_launch(GS, LDS, GF_THREADS * TPL, GF_THREADS);
     hipLaunchKernelGGL(kern, dim3((uint32_t)wgs), dim3(GF_THREADS), LDS, ctx->stream, d_idx,
                        reinterpret_cast<const float*>(a.d_lut), d_out, n, a.g.M, a.g.CB_pad, a.g.idx_row_bytes,
                        a.d_bias, a.d_scales, a.g.CB, a.desc.scale_group, a.desc.activation, n_token_tiles, by_xcd);
@@ -1191,15 +1194,19 @@ bool gather_dense_only()
 bool apply_runtime_tuning(AmmGeom* g, const pimdl_amm_tuning& t, std::string* why)
 {
     const bool matrix_core = g->gather_kind != 0;
-    if (t.token_item && (!matrix_core || (t.token_item != 128 && t.token_item != 256))) {
-        *why = "token_item must be 128 or 256, and only the matrix-core gathers (int8, up to 16 centroids) have it";
+    const bool eight_waves = t.token_item == 512 && g->gather_kind == 2;  // one workgroup of eight waves per CU
+    if (t.token_item && (!matrix_core || (t.token_item != 128 && t.token_item != 256 && !eight_waves))) {
+        *why = "token_item must be 128 or 256 (512 for the sparse kernel), and only the matrix-core gathers (int8, up to 16 centroids) have it";
         return false;
     }
     if (t.cb_per_slice) {
         const uint32_t entries = g->C_tile == 8 ? g->CB_pad / 2 : g->CB_pad;  // codebooks, or pairs of them
-        const bool has32 = g->gather_kind == 2 ? g->q <= 4 : (g->q == 3 || (g->q == 4 && g->C_tile != 8));
-        if (!matrix_core || (t.cb_per_slice != 16 && !(t.cb_per_slice == 32 && has32 && entries % 32 == 0))) {
-            *why = "cb_per_slice must be 16, or 32 where the operator's kernel has that variant";
+        const bool has32 = eight_waves || (g->gather_kind == 2 ? g->q <= 4 : (g->q == 3 || (g->q == 4 && g->C_tile != 8)));
+        const bool has64 = eight_waves && g->q == 3;
+        if (!matrix_core || (t.cb_per_slice == 16 && eight_waves && g->q == 3) ||
+            (t.cb_per_slice != 16 && !(t.cb_per_slice == 32 && has32 && entries % 32 == 0) &&
+                             !(t.cb_per_slice == 64 && has64 && entries % 64 == 0))) {
+            *why = "cb_per_slice must be 16, or 32 / 64 where the operator's kernel has that variant";
             return false;
         }
     }

@@ -53,14 +53,15 @@ namespace {
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v2i __attribute__((ext_vector_type(2)));
 
-constexpr int SP_WAVES = 4;
-constexpr int SP_THREADS = SP_WAVES * 64;
-constexpr int sp_tok_item(int tm) { return SP_WAVES * tm * 16; }
+// Waves per workgroup (NW): 4, two workgroups per CU -- or 8, one workgroup per CU: the same two waves per
+// SIMD, but a LUT slice is copied into LDS once for 512 tokens instead of 256 and the CU's whole LDS belongs
+// to one workgroup (slices twice as deep, half as many barriers).
+constexpr int sp_tok_item(int tm, int nw = 4) { return nw * tm * 16; }
 constexpr int sp_nbuf(int gs) { return gs > 16 ? 2 : 3; }
 constexpr int SP_TABLE = 256;  // 16 entries of 16 bytes
-constexpr int sp_lds_bytes(int tn, int gs)
+constexpr int sp_lds_bytes(int tn, int gs, int nw = 4)
 {
-    return SP_TABLE + sp_nbuf(gs) * gs * 16 * tn * 16 + sp_nbuf(gs) * SP_WAVES * 64 * 4 * (gs / 8);
+    return SP_TABLE + sp_nbuf(gs) * gs * 16 * tn * 16 + sp_nbuf(gs) * nw * 64 * 4 * (gs / 8);
 }
 
 template <int OFF>
@@ -83,13 +84,14 @@ __device__ __forceinline__ T* uniform_ptr(T* p)
     return reinterpret_cast<T*>(((uint64_t)hi << 32) | lo);
 }
 
-template <int TN, int TM, int GS>
-__global__ __launch_bounds__(SP_THREADS, 2) void gather_sparse_kernel(
+template <int TN, int TM, int GS, int NW>
+__global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel(
     const uint8_t* __restrict__ idx, const int8_t* __restrict__ lut, float* __restrict__ out,
     int32_t* __restrict__ acc_out, uint32_t N, uint32_t M, uint32_t CB_pad, uint32_t idx_row_bytes,
     uint32_t n_token_tiles, uint32_t n_items, Epilogue ep, XcdMap xmap)
 {
-    constexpr int TOK_ITEM = sp_tok_item(TM);
+    constexpr int SP_WAVES = NW;
+    constexpr int TOK_ITEM = sp_tok_item(TM, NW);
     static_assert(TM == 4 || TM == 2, "a wave owns a whole or half a 64-token index block");
     constexpr int WN = 16 * TN;                    // columns per item
     constexpr int G = GS;                          // codebooks per slice
@@ -436,14 +438,14 @@ __global__ __launch_bounds__(SP_THREADS, 2) void gather_sparse_kernel(
     }
 }
 
-template <int TN, int TM, int GS>
+template <int TN, int TM, int GS, int NW = 4>
 int launch_sparse_tm(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_t* d_acc, uint32_t n,
                      const Epilogue& ep)
 {
-    constexpr int LDS = sp_lds_bytes(TN, GS);
-    static_assert(2 * LDS <= 160 * 1024, "two workgroups per CU");
-    constexpr int TOK_ITEM = sp_tok_item(TM);
-    auto kern = gather_sparse_kernel<TN, TM, GS>;
+    constexpr int LDS = sp_lds_bytes(TN, GS, NW);
+    static_assert((NW == 4 ? 2 : 1) * LDS <= 160 * 1024, "two workgroups of four waves, or one of eight, per CU");
+    constexpr int TOK_ITEM = sp_tok_item(TM, NW);
+    auto kern = gather_sparse_kernel<TN, TM, GS, NW>;
     static bool attr_set = false;
     if (!attr_set) {
         int rc = hip_check(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -454,12 +456,13 @@ int launch_sparse_tm(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out,
     }
     const uint32_t n_token_tiles = (n + TOK_ITEM - 1) / TOK_ITEM;
     const uint32_t n_items = n_token_tiles * (a.g.M_pad / (16 * TN));
-    uint32_t grid = ctx->prop.multiProcessorCount * 2;
+    uint32_t grid = ctx->prop.multiProcessorCount * (NW == 4 ? 2 : 1);
     if (grid > n_items) grid = n_items;
     const XcdMap xmap = choose_xcd_map(a.g.M_pad / (16 * TN), n_token_tiles, grid, (uint64_t)a.g.CB_pad * 16 * a.g.M_pad,
                                        (uint64_t)n * a.g.idx_row_bytes, a.g.tune_xcd_col_split);
-    snprintf(a.last_gather, sizeof(a.last_gather), "gather_sparse_kernel<%d, %d, %d>", TN, TM, GS);
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(SP_THREADS), LDS, ctx->stream, d_idx, reinterpret_cast<const int8_t*>(a.d_lut),
+    snprintf(a.last_gather, sizeof(a.last_gather), "gather_sparse_kernel<%d, %d, %d, %d>", TN, TM, GS, NW);
+    a.note_launch(GS, LDS, TOK_ITEM, NW * 64);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), LDS, ctx->stream, d_idx, reinterpret_cast<const int8_t*>(a.d_lut),
                        d_out, d_acc, n, a.g.M, a.g.CB_pad, a.g.idx_row_bytes, n_token_tiles, n_items, ep, xmap);
     return hip_check(ctx, hipGetLastError(), "gather_sparse_kernel launch");
 }
@@ -474,6 +477,26 @@ int launch_sparse_tn(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out,
     const uint64_t slots = 2ull * ctx->prop.multiProcessorCount;
     bool small_items = items4 < slots || 10 * ((items2 + slots - 1) / slots) < 17 * ((items4 + slots - 1) / slots);
     if (a.g.tune_token_item) small_items = a.g.tune_token_item == 128;
+    // 48-column tiles read the sparse operand of a token group for three column groups only, so the copies and
+    // the per-slice costs weigh most there: with eight waves per workgroup a slice is copied once per 512 tokens
+    // and can be 64 codebooks deep (measured 44.1 -> 42.4 us at 3072 -> 768, N = 8192; the 96-column kernel
+    // loses 3 us the same way, its two waves of a SIMD then waiting at the same barrier).  Taken where it costs
+    // no extra round of the grid and still gives every CU a workgroup.
+    if constexpr (TN == 3) {
+        const uint64_t cus = ctx->prop.multiProcessorCount;
+        const uint64_t items8 = (uint64_t)((n + sp_tok_item(4, 8) - 1) / sp_tok_item(4, 8)) * col_tiles;
+        if (!a.g.tune_token_item && !a.g.tune_cb_per_slice && a.g.CB_pad % 64 == 0 && !small_items && items8 >= cus &&
+            (items8 + cus - 1) / cus <= (items4 + slots - 1) / slots)
+            return launch_sparse_tm<TN, 4, 64, 8>(ctx, a, d_idx, d_out, d_acc, n, ep);
+    }
+    if (a.g.tune_token_item == 512) {  // one workgroup of eight waves per CU
+        if constexpr (TN == 3) {
+            if (a.g.CB_pad % 64 == 0 && a.g.tune_cb_per_slice == 64) return launch_sparse_tm<TN, 4, 64, 8>(ctx, a, d_idx, d_out, d_acc, n, ep);
+        }
+        // (CB_pad is a multiple of 32; 48-column tiles have no 16-codebook variant here: 12 blocks for 8 waves)
+        if (TN == 3 || a.g.tune_cb_per_slice != 16) return launch_sparse_tm<TN, 4, 32, 8>(ctx, a, d_idx, d_out, d_acc, n, ep);
+        if constexpr (TN != 3) return launch_sparse_tm<TN, 4, 16, 8>(ctx, a, d_idx, d_out, d_acc, n, ep);
+    }
     constexpr int GSB = TN <= 4 ? 32 : 16;  // 32-codebook slices in two buffers where two workgroups still fit a CU
     if constexpr (GSB != 16) {
         if (a.g.CB_pad % GSB == 0 && a.g.tune_cb_per_slice != 16) {

@@ -945,10 +945,13 @@ int pimdl_amm_get_geometry(const pimdl_amm* a, pimdl_amm_geometry* out)
     out->idx_row_bytes = g.idx_row_bytes;
     out->col_block = g.col_block;
     out->row_pitch = g.row_pitch;
-    out->cb_per_slice = g.cb_per_slice;
-    out->lds_bytes = g.gather_lds_bytes;
-    out->tokens_per_wg = g.tokens_per_wg;
-    out->gather_threads = g.gather_threads;
+    // the gather launcher picks among instances of its kernel by the batch it is given: report the last launch's
+    // shape once there has been one, the plan's defaults before
+    const bool ran = a->last_threads != 0;
+    out->cb_per_slice = ran ? a->last_cb_per_slice : g.cb_per_slice;
+    out->lds_bytes = ran ? a->last_lds_bytes : g.gather_lds_bytes;
+    out->tokens_per_wg = ran ? a->last_tokens_per_wg : g.tokens_per_wg;
+    out->gather_threads = ran ? a->last_threads : g.gather_threads;
     out->ccs_tokens_per_wg = 64;
     out->ccs_cb_per_wg = g.ccs_cb_per_wg;
     out->ccs_threads = 256;

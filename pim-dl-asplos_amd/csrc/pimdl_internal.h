@@ -84,6 +84,15 @@ struct Amm {
     uint32_t op_col_tiles, op_idx_stride;
     // name (with template arguments) of the gather kernel the operator's last launch used: what a profile lists
     mutable char last_gather[80];
+    // shape of that launch (0 before the first one): codebooks per slice, LDS bytes, tokens and threads per workgroup
+    mutable uint32_t last_cb_per_slice = 0, last_lds_bytes = 0, last_tokens_per_wg = 0, last_threads = 0;
+    void note_launch(uint32_t cb_per_slice, uint32_t lds_bytes, uint32_t tokens_per_wg, uint32_t threads) const
+    {
+        last_cb_per_slice = cb_per_slice;
+        last_lds_bytes = lds_bytes;
+        last_tokens_per_wg = tokens_per_wg;
+        last_threads = threads;
+    }
 };
 
 struct Ctx {

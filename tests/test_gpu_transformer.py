@@ -384,6 +384,9 @@ def test_every_tuning_choice_gives_the_same_bits(ctx):
             settings += [{"cb_per_slice": 16}, {"token_item": 128, "cb_per_slice": 16, "xcd_col_split": 2}]
             if cb <= 64:
                 settings.append({"cb_per_slice": 32})
+            if gk == pimdl.GATHER_SPARSE:  # one workgroup of eight waves per CU: 512-token items
+                settings += [{"token_item": 512}, {"token_item": 512, "cb_per_slice": 32, "xcd_col_split": 4}]
+                settings.append({"token_item": 512, "cb_per_slice": 64} if cb == 48 else {"token_item": 512, "cb_per_slice": 16})
         settings += [{"search_kernel": k} for k in (1, 2, 3)] + [{"search_kernel": 3, "search_token_tile": t} for t in (64, 128)]
         for st in settings:
             amm.set_tuning(**st)
@@ -393,6 +396,11 @@ def test_every_tuning_choice_gives_the_same_bits(ctx):
         if gk != pimdl.GATHER_ROWS and cb == 96:
             with pytest.raises(pimdl.PimdlError):
                 amm.set_tuning(cb_per_slice=32)
+            with pytest.raises(pimdl.PimdlError):
+                amm.set_tuning(token_item=512, cb_per_slice=64)
+        if gk == pimdl.GATHER_ONEHOT:
+            with pytest.raises(pimdl.PimdlError):
+                amm.set_tuning(token_item=512)
         with pytest.raises(pimdl.PimdlError):
             amm.set_tuning(col_block=48 if cb != 48 else 64)
         with pytest.raises(pimdl.PimdlError):
