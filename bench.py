@@ -92,6 +92,63 @@ def model_forward(pimdl, ctx, iters=10):
             "note": "LUT-AMM linears (tanh-GELU inside the first feed-forward operator's epilogue), pimdl_layer_norm and pimdl_attention (fp32) on libpimdl; PyTorch-ROCm for tensors, streams and graph capture"}
 
 
+def bert_large_layer(pimdl, ctx, iters=20):
+    """One BERT-large encoder layer as a layer (hidden 1024, 16 heads x 64, feed-forward 4096, N = 64 x 128 = 8192
+    tokens, every linear a LUT-AMM with v=4, C=16, int8 LUTs): time of the whole layer and of each of its stages
+    launched on its own (device time between two events around `iters` launches, after the clock has settled)."""
+    import torch
+    from pim_dl_asplos_amd import transformer as T
+    p = T.TransformerParams(128, 64, 16, 64, 1024, 4096, 1)
+    for op, (k_in, m_out) in {"q": (1024, 1024), "k": (1024, 1024), "v": (1024, 1024), "o": (1024, 1024),
+                              "ffn1": (1024, 4096), "ffn2": (4096, 1024)}.items():
+        p.shapes[op] = T.AmmShape(k_in // 4, 16, k_in, m_out)
+    layer = T.TransformerLayer(ctx, pimdl, T.synth_layers(p, ctx, pimdl, seed=2)[0], p)
+    n, d = p.n, p.token_dim
+    x = torch.randn((n, d), device="cuda", dtype=torch.float32)
+    keep = {}
+    layer.forward(x, keep)
+
+    def timed(fn, reps):
+        t_end = time.perf_counter() + 0.03          # about 30 ms of the same work first: clock ramp
+        while time.perf_counter() < t_end:
+            fn()
+            torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    ms_layer = timed(lambda: layer.forward(x), iters)
+    qkv = torch.empty((n, 3 * d), device="cuda", dtype=torch.float32)
+    out_d = torch.empty((n, d), device="cuda", dtype=torch.float32)
+    out_f = torch.empty((n, p.ffn_hidden_dim), device="cuda", dtype=torch.float32)
+    q, k, v = (qkv[:, i * d:(i + 1) * d] for i in range(3))
+    w1, b1 = layer.norm["attention_norm"]
+    stages = {}
+    if layer.qkv_group is not None and layer.qkv_group.fused_cols == 3 * d:
+        stages["qkv (one search, one gather into [q|k|v])"] = lambda: layer.qkv_group.run_fused_ptr(x.data_ptr(), n, qkv.data_ptr())
+    for i, name in enumerate(("q", "k", "v")):   # the attention stage reads this layer's own projections
+        qkv[:, i * d:(i + 1) * d].copy_(keep[name])
+    stages["attention"] = lambda: ctx.attention_ptr(q.data_ptr(), k.data_ptr(), v.data_ptr(), out_d.data_ptr(), p.batch_size,
+                                                    p.seq_len, p.head_num, p.head_dim, q.stride(0), d, 0.125)
+    stages["o"] = lambda: layer.amm["o"].run_ptr(keep["attn"].data_ptr(), n, out_d.data_ptr())
+    stages["attention_norm (+ residual)"] = lambda: ctx.layer_norm((keep["o"].data_ptr(), n, d), w1.data_ptr(), b1.data_ptr(),
+                                                                   x.data_ptr(), out_d.data_ptr(), 1e-6)
+    stages["ffn1 (+ GELU in the epilogue)"] = lambda: layer.amm["ffn1"].run_ptr(keep["h"].data_ptr(), n, out_f.data_ptr())
+    stages["ffn2"] = lambda: layer.amm["ffn2"].run_ptr(keep["gelu"].data_ptr(), n, out_d.data_ptr())
+    stages["ffn_norm (+ residual)"] = lambda: ctx.layer_norm((keep["ffn2"].data_ptr(), n, d), w1.data_ptr(), b1.data_ptr(),
+                                                             keep["h"].data_ptr(), out_d.data_ptr(), 1e-6)
+    per_stage = {name: round(timed(fn, iters) * 1e3, 1) for name, fn in stages.items()}
+    layer.close()
+    return {"tokens": n, "token_dim": d, "head_num": p.head_num, "ffn_hidden_dim": p.ffn_hidden_dim,
+            "ms_per_layer": ms_layer, "tokens_per_s": n / (ms_layer * 1e-3), "stage_us": per_stage,
+            "note": "stages launched on their own; their sum exceeds the layer's time by the per-launch hand-overs "
+                    "that back-to-back kernels of the layer hide"}
+
+
 def cpu_baseline(shapes, N, warmup=10, rounds=20, budget_s=25.0):
     """The oracle's restatement of the reference's amm_cpu (test_amm.cpp:126-183) on this host's cores, on the
     full batch of both AMMs, with the reference driver's protocol (test_amm.cpp:21-22,290-314: 10 warm-up and
@@ -363,6 +420,7 @@ def main():
                               "note": "pageable host memory in and out of both AMMs (PCIe copies included), 3 steps"}
     if not args.no_model:
         result["bert_base_forward"] = model_forward(pimdl, ctx)
+        result["bert_large_layer"] = bert_large_layer(pimdl, ctx)
     if not args.no_sweep:
         result["per_codebook_scale"] = per_codebook_scale(pimdl, ctx, rng, N, shapes)
         result["vit_base_sweep"] = vit_sweep(pimdl, ctx)
