@@ -145,8 +145,8 @@ def bert_large_layer(pimdl, ctx, iters=20):
     layer.close()
     return {"tokens": n, "token_dim": d, "head_num": p.head_num, "ffn_hidden_dim": p.ffn_hidden_dim,
             "ms_per_layer": ms_layer, "tokens_per_s": n / (ms_layer * 1e-3), "stage_us": per_stage,
-            "note": "stages launched on their own; their sum exceeds the layer's time by the per-launch hand-overs "
-                    "that back-to-back kernels of the layer hide"}
+            "note": "ms_per_layer: the whole forward, launched op by op from Python; stage_us: each stage launched on "
+                    "its own, back to back with itself (inputs warm in the caches, no allocation between launches)"}
 
 
 def cpu_baseline(shapes, N, warmup=10, rounds=20, budget_s=25.0):

@@ -24,6 +24,30 @@ struct Epilogue {
     uint32_t op_col_tiles, op_idx_stride;
 };
 
+// Time of a launch whose persistent grid of `slots` workgroups (two per CU) shares `items` equal items, in units
+// of a full round.  Whole rounds cost 1 each.  A partly filled round costs less than a full one, because a
+// workgroup that has a CU to itself runs faster (one item per CU: 0.65 of the time two per CU take, measured with
+// the sparse kernel's 256-token items at 768 -> 3072: 256 items 13.7 us, 512 items 20.9 us after the launch's
+// fixed 4.4 us), and after the first round the stragglers of a round also overlap with the round before
+// (640 items 1.40, 768 items 1.48, 1024 items 2.0 rounds).
+inline double grid_rounds(uint64_t items, uint64_t slots)
+{
+    const uint64_t full = items / slots, rem = items % slots;
+    if (rem == 0) return (double)full;
+    if (2 * rem > slots) return (double)full + 0.9;
+    return (double)full + (full == 0 ? 0.65 : 0.5);
+}
+// Time of one item of the matrix-core gathers relative to a 256-token x 96-column one (same number of codebooks):
+// 64- and 48-column tiles read the one-hot operand for fewer column groups (measured per round at 768 -> 3072,
+// N = 8192, launch overhead taken off: 21.5 / 14.7 / 13.1 us; 27.9 / 19.2 at 1024 -> 4096); a 128-token item takes
+// 0.62 of a 256-token one.
+inline double item_cost(uint32_t tn, bool small_item) { return (tn >= 6 ? 1.0 : tn == 4 ? 0.70 : 0.61) * (small_item ? 0.62 : 1.0); }
+// 128-token items instead of 256-token ones where that is the shorter launch by the two figures above.
+inline bool prefer_small_items(uint64_t items256, uint64_t items128, uint64_t slots)
+{
+    return grid_rounds(items128, slots) * 0.62 < grid_rounds(items256, slots);
+}
+
 // How the items (column tile x token tile) of a gather are dealt to the 8 XCDs.  Workgroup b takes
 // positions b, b + grid, ... of the item sequence and the hardware places workgroups on the XCDs
 // round-robin, so (for a grid that is a multiple of 8) positions congruent mod 8 run on one XCD, each

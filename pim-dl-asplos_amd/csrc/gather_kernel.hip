@@ -834,10 +834,9 @@ int launch_onehot_tm(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out,
     return hip_check(ctx, hipGetLastError(), "gather_onehot_kernel launch");
 }
 
-// 256-token items (TM = 4) need fewer LDS reads and copies per MFMA; when the batch does not offer
-// two of them per CU, 128-token items (TM = 2) put a second wave on every SIMD instead.  In between the
-// item size that needs the shorter time wins: rounds of the persistent grid x the cost of an item (a
-// 256-token item takes 1.7 times as long as a 128-token one).
+// 256-token items (TM = 4) need fewer LDS reads and copies per MFMA; 128-token items (TM = 2) fill the grid
+// of a small batch better.  The item size that needs the shorter time wins: rounds of the persistent grid,
+// partly filled ones counted for what they cost (grid_rounds), x the cost of an item.
 template <int TN, bool P8>
 int launch_onehot(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_t* d_acc, uint32_t n,
                   const Epilogue& ep)
@@ -849,7 +848,7 @@ int launch_onehot(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, in
     constexpr int GSB = (TN == 3 || (TN == 4 && !P8)) ? 32 : 16;
     const uint64_t slots = 2ull * ctx->prop.multiProcessorCount;
     const uint64_t items2 = (uint64_t)((n + oh_tok_item(2) - 1) / oh_tok_item(2)) * (a.g.M_pad / (16 * TN));
-    bool small_items = items4 < slots || 10 * ((items2 + slots - 1) / slots) < 17 * ((items4 + slots - 1) / slots);
+    bool small_items = prefer_small_items(items4, items2, slots);
     if (a.g.tune_token_item) small_items = a.g.tune_token_item == 128;
     if constexpr (GSB != 16) {
         const uint32_t entries = P8 ? a.g.CB_pad / 2 : a.g.CB_pad;
@@ -1277,16 +1276,16 @@ bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::s
     }
     g->idx_tiled = g->gather_kind != 0;
     if (g->gather_kind != 0) {
-        // One-hot matrix-core kernel: an item is 256 tokens x 16*TN columns, all items cost the
-        // same.  Take the TN that fills the persistent grid (two workgroups per CU) most evenly for
-        // the largest batch this operator will see; among equals the widest (fewest LDS reads).
+        // One-hot matrix-core kernel: an item is 256 tokens x 16*TN columns.  Take the TN with the shortest
+        // launch for the largest batch this operator will see: rounds of the persistent grid (two workgroups
+        // per CU; grid_rounds) x the cost of an item of that width; among equals the widest.
         // up to 8 centroids: two codebooks share a lane's 16 K-slots (C_tile 8); 96-column tiles then do not
         // leave room for two workgroups per CU
         const bool paired = C <= 8;
         g->C_tile = paired ? 8 : 16;
         const uint32_t slots = 2 * (num_cus ? num_cus : 256);
         const uint32_t tiles = (d.max_n + 255) / 256;
-        double best = -1.0;
+        double best = 1e300;
         if (col_block_hint && col_block_hint != 64 && col_block_hint != 48 && (paired || col_block_hint != 96)) {
             *why = paired ? "column tile hint must be 48 or 64 for this operator"
                           : "column tile hint must be 48, 64 or 96 for this operator";
@@ -1297,10 +1296,12 @@ bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::s
             if (col_block_hint && col_block_hint != 16 * tn) continue;
             const uint32_t blocks = (M + 16 * tn - 1) / (16 * tn);
             const uint64_t items = (uint64_t)tiles * blocks;
-            const uint64_t rounds = (items + slots - 1) / slots;
-            const double eff = (double)items / (double)(rounds * slots) * (double)M / (double)(blocks * 16 * tn);
-            if (eff > best + 1e-9) {
-                best = eff;
+            const uint64_t items_small = (uint64_t)((d.max_n + 127) / 128) * blocks;
+            const double t256 = grid_rounds(items, slots) * item_cost(tn, false);
+            const double t128 = grid_rounds(items_small, slots) * item_cost(tn, true);
+            const double t = t128 < t256 ? t128 : t256;  // the launcher takes the better item size
+            if (t < best - 1e-9) {
+                best = t;
                 g->q = tn;
             }
         }

@@ -467,7 +467,7 @@ int launch_sparse_tm(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out,
     return hip_check(ctx, hipGetLastError(), "gather_sparse_kernel launch");
 }
 
-// 256-token items where the batch offers two of them per CU, else 128-token items (the rule of the dense kernel)
+// 256- or 128-token items, whichever gives the shorter launch (the rule of the dense kernel)
 template <int TN>
 int launch_sparse_tn(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_t* d_acc, uint32_t n, const Epilogue& ep)
 {
@@ -475,7 +475,7 @@ int launch_sparse_tn(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out,
     const uint64_t items4 = (uint64_t)((n + sp_tok_item(4) - 1) / sp_tok_item(4)) * col_tiles;
     const uint64_t items2 = (uint64_t)((n + sp_tok_item(2) - 1) / sp_tok_item(2)) * col_tiles;
     const uint64_t slots = 2ull * ctx->prop.multiProcessorCount;
-    bool small_items = items4 < slots || 10 * ((items2 + slots - 1) / slots) < 17 * ((items4 + slots - 1) / slots);
+    bool small_items = prefer_small_items(items4, items2, slots);
     if (a.g.tune_token_item) small_items = a.g.tune_token_item == 128;
     // 48-column tiles read the sparse operand of a token group for three column groups only, so the copies and
     // the per-slice costs weigh most there: with eight waves per workgroup a slice is copied once per 512 tokens
