@@ -773,6 +773,9 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
     // A wave's priority falls as its workgroup progresses through its share: whoever is behind goes first.
     const uint32_t my_tiles = (total_tiles - blockIdx.x + gridDim.x - 1) / gridDim.x;
     uint32_t tiles_done = 0;
+    uint32_t tcb_loaded = 0xFFFFFFFFu;  // codebook tile whose operands are resident (registers and LDS)
+    uint4 aq[2][NM];
+    float cmax[2];
     for (uint32_t tile_id = blockIdx.x; tile_id < total_tiles; tile_id += gridDim.x) {
         switch (4 * tiles_done / my_tiles) {
             case 0: __builtin_amdgcn_s_setprio(3); break;
@@ -785,28 +788,34 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
         const uint32_t tcb = tile_id % tiles_cb;          // codebooks 16 tcb .. 16 tcb + 15
         const uint32_t pair0 = tcb * (CBW / 2) + 2 * wave;  // first of this wave's two pairs
 
-        uint4 aq[2][NM];
+        // What depends on the codebooks alone stays from the previous tile when this one has the same codebooks
+        // (a grid that is a multiple of the codebook tiles gives a workgroup the same ones every time).
+        const bool new_cb = tcb != tcb_loaded;  // workgroup-uniform
+        tcb_loaded = tcb;
+        if (new_cb) {
 #pragma unroll
-        for (int pl = 0; pl < 2; ++pl)
+            for (int pl = 0; pl < 2; ++pl)
 #pragma unroll
-            for (int m = 0; m < NM; ++m) aq[pl][m] = aux_b[((size_t)(pair0 + pl) * NM + m) * 64 + lane];
-        // every global load the search needs is issued here, ahead of the next tile's prefetch:
-        // loads complete in order, so a later load would have to wait for the prefetch from HBM
-        float cmax[2];
+                for (int m = 0; m < NM; ++m) aq[pl][m] = aux_b[((size_t)(pair0 + pl) * NM + m) * 64 + lane];
+            // every global load the search needs is issued here, ahead of the next tile's prefetch:
+            // loads complete in order, so a later load would have to wait for the prefetch from HBM
 #pragma unroll
-        for (int pl = 0; pl < 2; ++pl) cmax[pl] = cnmax_pad[WIDE ? pair0 + pl : 2 * (pair0 + pl) + h];
-        // raw centroids of the tile's codebooks, only read by exact replays
-        const uint32_t cb_here = (CB - tcb * RCB < (uint32_t)RCB) ? CB - tcb * RCB : (uint32_t)RCB;
-        const uint32_t cent_fl = cb_here * C * V;
-        const float* csrc = cent + (size_t)tcb * RCB * C * V;  // 16-byte aligned: RCB * V * 4 bytes per c
+            for (int pl = 0; pl < 2; ++pl) cmax[pl] = cnmax_pad[WIDE ? pair0 + pl : 2 * (pair0 + pl) + h];
+        }
 #pragma unroll
         for (int i = 0; i < PASSES; ++i)
             *reinterpret_cast<float4*>(&tile[(fr0 + i * ROWS_PER_PASS) * PITCH + 4 * fq]) = pf[i];
-        for (uint32_t i = threadIdx.x; i < cent_fl / 4; i += CCS_THREADS)
-            reinterpret_cast<float4*>(cst)[i] = reinterpret_cast<const float4*>(csrc)[i];
-        if (threadIdx.x < cent_fl % 4) cst[cent_fl - 1 - threadIdx.x] = csrc[cent_fl - 1 - threadIdx.x];
-        if (threadIdx.x < CBW * 16 / 4)
-            reinterpret_cast<float4*>(cnl)[threadIdx.x] = reinterpret_cast<const float4*>(cn16 + (size_t)tcb * CBW * 16)[threadIdx.x];
+        if (new_cb) {
+            // raw centroids of the tile's codebooks, only read by exact replays
+            const uint32_t cb_here = (CB - tcb * RCB < (uint32_t)RCB) ? CB - tcb * RCB : (uint32_t)RCB;
+            const uint32_t cent_fl = cb_here * C * V;
+            const float* csrc = cent + (size_t)tcb * RCB * C * V;  // 16-byte aligned: RCB * V * 4 bytes per c
+            for (uint32_t i = threadIdx.x; i < cent_fl / 4; i += CCS_THREADS)
+                reinterpret_cast<float4*>(cst)[i] = reinterpret_cast<const float4*>(csrc)[i];
+            if (threadIdx.x < cent_fl % 4) cst[cent_fl - 1 - threadIdx.x] = csrc[cent_fl - 1 - threadIdx.x];
+            if (threadIdx.x < CBW * 16 / 4)
+                reinterpret_cast<float4*>(cnl)[threadIdx.x] = reinterpret_cast<const float4*>(cn16 + (size_t)tcb * CBW * 16)[threadIdx.x];
+        }
         __syncthreads();
         if (tile_id + gridDim.x < total_tiles) fetch(pf, tile_id + gridDim.x);
 
@@ -816,10 +825,10 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
         // pieces of -2c, and the K-slots pair them as  xh*ch, xh*cm, xm*ch, xm*cm, xh*cl, xl*ch  (the three
         // omitted products are below 2^-20 |x||c|).  Products of bf16 values are exact in fp32; the
         // accumulators start from |c|^2.  xx_out: |x|^2 over the lane's own codebook (for the bound).
-        auto scores = [&](floatx16& acc, float& xx_out, int it) {
+        // activations of item `it` for this lane; read two items ahead of their use (see the loop below)
+        auto load_x = [&](float (&xs)[2][DL], int it) {
             const int pl = it / TG, tg = it % TG;
             const float* brow = brow0 + tg * 32 * PITCH + pl * XSTEP;
-            float xs[2][DL];
 #pragma unroll
             for (int cbh = 0; cbh < 2; ++cbh) {
                 const float* src = brow + (WIDE ? 0 : cbh * V) + DL * h;
@@ -838,14 +847,20 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
                     xs[cbh][3] = t4.w;
                 }
             }
-            const float4* cnp = reinterpret_cast<const float4*>(cnl + (2 * (2 * wave + pl) + h) * 16);
+        };
+        floatx16 cn_pl;  // |c|^2 of the lane's 16 centroids of the current pair: what every accumulator starts from
+        auto scores = [&](floatx16& acc, float& xx_out, int it, const float (&xs)[2][DL]) {
+            const int pl = it / TG;
+            if (it % TG == 0) {  // (a constant once the item loop is unrolled) first token group of a pair
+                const float4* cnp = reinterpret_cast<const float4*>(cnl + (2 * (2 * wave + pl) + h) * 16);
 #pragma unroll
-            for (int q4 = 0; q4 < 4; ++q4) {
-                const float4 c4 = cnp[q4];
-                acc[4 * q4 + 0] = c4.x;
-                acc[4 * q4 + 1] = c4.y;
-                acc[4 * q4 + 2] = c4.z;
-                acc[4 * q4 + 3] = c4.w;
+                for (int q4 = 0; q4 < 4; ++q4) {
+                    const float4 c4 = cnp[q4];
+                    cn_pl[4 * q4 + 0] = c4.x;
+                    cn_pl[4 * q4 + 1] = c4.y;
+                    cn_pl[4 * q4 + 2] = c4.z;
+                    cn_pl[4 * q4 + 3] = c4.w;
+                }
             }
             uint32_t breg[NM * 4];
 #pragma unroll
@@ -892,7 +907,7 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
 #pragma unroll
             for (int m = 0; m < NM; ++m) {
                 const uint4 bm = make_uint4(breg[4 * m], breg[4 * m + 1], breg[4 * m + 2], breg[4 * m + 3]);
-                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, aq[pl][m]), __builtin_bit_cast(bf16x8, bm), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, aq[pl][m]), __builtin_bit_cast(bf16x8, bm), m == 0 ? cn_pl : acc, 0, 0, 0);
             }
         };
 
@@ -904,12 +919,22 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
 
         floatx16 acc_cur, acc_nxt;
         float xx_cur, xx_nxt;
-        scores(acc_cur, xx_cur, 0);
+        // The activations of item it + 2 are read from LDS before item it + 1 is scored and item it searched, and
+        // the read is kept there: left to itself the compiler sinks it to a few instructions before its use and
+        // the wave waits out the LDS latency once per item.
+        float xs_ring[3][2][DL];
+        load_x(xs_ring[0], 0);
+        if constexpr (ITEMS > 1) load_x(xs_ring[1], 1);
+        scores(acc_cur, xx_cur, 0, xs_ring[0]);
         static_for<ITEMS>([&](auto itc) {
             constexpr int it = decltype(itc)::value;
             constexpr int pl = it / TG, tg = it % TG;
             (void)tg;
-            if constexpr (it + 1 < ITEMS) scores(acc_nxt, xx_nxt, it + 1);
+            if constexpr (it + 2 < ITEMS) {
+                load_x(xs_ring[(it + 2) % 3], it + 2);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if constexpr (it + 1 < ITEMS) scores(acc_nxt, xx_nxt, it + 1, xs_ring[(it + 1) % 3]);
             const float xx = xx_cur;
             // smallest (m1) and second smallest (m2) of the 16 id-tagged scores, 36 VALU operations:
             // five triples give (min3, med3) each; the overall second smallest is the smaller of
@@ -1192,7 +1217,11 @@ int launch_ccs_bf16_tt(Ctx* ctx, const AmmGeom& g, const float* d_x, const float
         per_cu = q;
     }
     const uint32_t slots = (uint32_t)ctx->prop.multiProcessorCount * (uint32_t)per_cu;
-    dim3 grid(total < slots ? total : slots);
+    uint32_t grid_wgs = total < slots ? total : slots;
+    // a grid that is a multiple of the codebook tiles gives every workgroup the same codebooks tile after tile,
+    // and the kernel then keeps their operands; taken where it costs at most 4 % of the resident workgroups
+    if (total > slots && tiles_cb <= slots && (slots / tiles_cb) * tiles_cb * 25 >= slots * 24) grid_wgs = (slots / tiles_cb) * tiles_cb;
+    dim3 grid(grid_wgs);
     const uint32_t row = x_cols ? x_cols : g.K;  // floats per activation row
     const uint32_t tiles_x = x_cols ? x_cols / S::TF : tiles_cb;
     const int vec_ok = (row % 4 == 0) && ((reinterpret_cast<uintptr_t>(d_x) & 15) == 0);
@@ -1214,9 +1243,11 @@ int launch_ccs_bf16(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d
                     uint32_t x_cols)
 {
     const uint64_t tiles128 = (uint64_t)((n + 127) / 128) * (g.CB_pad / CcsMfmaShape<V, WIDE>::RCB);
-    // (measured: 7.4 -> 5.9 us at 192 tiles, 8.7 -> 6.9 us at 384, equal at 768 = one per resident workgroup,
-    // 10 % slower beyond)
-    const bool small_tiles = g.tune_search_tile ? g.tune_search_tile == 64 : tiles128 < 3ull * ctx->prop.multiProcessorCount;
+    // 64-token tiles up to two 128-token tiles per resident workgroup: four workgroups fit a CU instead of three,
+    // and since a workgroup keeps the operands of its codebooks from tile to tile the extra tiles cost little
+    // (measured 64 / 128-token tiles, us: 6.1 / 8.7 at 192 tiles; 11.0 / 11.9 at 768; 14.8 / 15.5 at 1188;
+    // 17.8 / 18.8 at 1536; 28.2 .. 31.5 / 28.2 .. 29.0 at 3072; 42.3 / 41.8 at 4752)
+    const bool small_tiles = g.tune_search_tile ? g.tune_search_tile == 64 : tiles128 <= 6ull * ctx->prop.multiProcessorCount;
     if (small_tiles) return launch_ccs_bf16_tt<V, WIDE, 64>(ctx, g, d_x, d_cent, d_idx, n, x_cols);
     return launch_ccs_bf16_tt<V, WIDE, 128>(ctx, g, d_x, d_cent, d_idx, n, x_cols);
 }
