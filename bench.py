@@ -202,7 +202,8 @@ def per_codebook_scale(pimdl, ctx, rng, N, shapes, iters=20):
     """The same pair with one fp32 scale per codebook (scale_group = 1), the wording of the benchmark
     configuration; the reference itself has one scale per tensor, which is what `value` measures.  A different
     scale per codebook rules out integer accumulation across codebooks: the table is resident as fp32 integers
-    and gathered by the fp32-table kernel (VALU adds), so this mode runs at that kernel's rate."""
+    (already multiplied by its codebook's scale: one rounding, as the definition has it) and gathered by the
+    fp32-table kernel (VALU adds), so this mode runs at that kernel's rate."""
     import torch
     out = []
     for (K, v, C, M) in shapes:

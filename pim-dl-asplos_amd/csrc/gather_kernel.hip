@@ -1153,7 +1153,7 @@ int launch_f32_tpl(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, u
 template <int C_T, int Q, int GS, int IDX_BITS>
 int launch_f32(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, uint32_t n)
 {
-    return a.grouped ? launch_f32_tpl<C_T, Q, GS, IDX_BITS, true>(ctx, a, d_idx, d_out, n)
+    return a.grouped && !a.prescaled ? launch_f32_tpl<C_T, Q, GS, IDX_BITS, true>(ctx, a, d_idx, d_out, n)
                      : launch_f32_tpl<C_T, Q, GS, IDX_BITS, false>(ctx, a, d_idx, d_out, n);
 }
 

@@ -386,6 +386,7 @@ int pimdl_amm_create_with(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const floa
     a->d_scales = nullptr;
     a->d_bias = nullptr;
     a->grouped = grouped;
+    a->prescaled = grouped && desc->scale_group == 1;
     a->d_op_scales = nullptr;
     a->op_col_tiles = 0;
     a->op_idx_stride = 0;
@@ -410,6 +411,17 @@ int pimdl_amm_create_with(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const floa
         try {
             const int8_t* q = reinterpret_cast<const int8_t*>(lut);
             wide.assign(q, q + (size_t)g.CB * g.C * g.M);  // int8 -> float, exact
+            if (a->prescaled) {
+                // one scale per codebook: a group's sum is the entry itself, so scaling it here (one fp32
+                // rounding) is what the kernel would do at every group boundary, and the adds that remain are
+                // those of an fp32 table in the same order
+                const size_t per_cb = (size_t)g.C * g.M;
+                for (uint32_t cb = 0; cb < g.CB; ++cb) {
+                    const float sc = scales[cb];
+                    float* w = wide.data() + cb * per_cb;
+                    for (size_t i = 0; i < per_cb; ++i) w[i] = w[i] * sc;
+                }
+            }
         } catch (...) {
             delete a;
             return set_error(ctx, PIMDL_ERR_NOMEM, "pimdl_amm_create: host staging of the widened table failed");

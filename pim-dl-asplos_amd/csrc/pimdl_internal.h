@@ -79,6 +79,8 @@ struct Amm {
     float* d_bias;       // [M]
     float h_scale0;
     bool grouped;        // int8 LUT with scale_group > 0: resident as fp32 integers, fp32 gather kernel
+    bool prescaled;      // ... with scale_group == 1: resident already multiplied by its codebook's scale (the one
+                         // rounding the grouped kernel would apply per entry), gathered like an fp32 table: same bits
     // several one-hot operators laid side by side along the columns (see Epilogue in gather_kernel.hip)
     float* d_op_scales;
     uint32_t op_col_tiles, op_idx_stride;
