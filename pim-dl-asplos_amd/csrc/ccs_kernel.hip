@@ -746,20 +746,29 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
     const uint32_t fr0 = threadIdx.x / F4_PER_ROW;
     auto fetch = [&](float4 (&pf)[PASSES], uint32_t tile_id) {
         const uint32_t t_tok0 = (tile_id / tiles_cb) * TT;
-        const uint32_t col = ((tile_id % tiles_cb) % tiles_x) * TF + 4 * fq;
+        const uint32_t col0 = ((tile_id % tiles_cb) % tiles_x) * TF;  // workgroup-uniform
+        const uint32_t col = col0 + 4 * fq;
+        // The whole tile inside the row and 16-byte aligned (every tile but a ragged last one): one 16-byte load
+        // per pass, decided once for the workgroup.  Decided per lane instead, the compiler splits every load in
+        // two and wraps each pass in a dozen exec-mask operations.
+        if (vec_ok && col0 + TF <= K) {
+#pragma unroll
+            for (int i = 0; i < PASSES; ++i) {
+                uint32_t tok = t_tok0 + fr0 + i * ROWS_PER_PASS;
+                tok = tok < N ? tok : N - 1;  // rows past N repeat the last token; never stored
+                pf[i] = *reinterpret_cast<const float4*>(x + (size_t)tok * K + col);
+            }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < PASSES; ++i) {
             uint32_t tok = t_tok0 + fr0 + i * ROWS_PER_PASS;
-            if (tok >= N) tok = N - 1;  // rows past N repeat the last token; never stored
+            if (tok >= N) tok = N - 1;
             const float* src = x + (size_t)tok * K + col;
-            if (vec_ok && col + 4 <= K) {
-                pf[i] = *reinterpret_cast<const float4*>(src);
-            } else {
-                pf[i].x = (col + 0 < K) ? src[0] : 0.0f;
-                pf[i].y = (col + 1 < K) ? src[1] : 0.0f;
-                pf[i].z = (col + 2 < K) ? src[2] : 0.0f;
-                pf[i].w = (col + 3 < K) ? src[3] : 0.0f;
-            }
+            pf[i].x = (col + 0 < K) ? src[0] : 0.0f;
+            pf[i].y = (col + 1 < K) ? src[1] : 0.0f;
+            pf[i].z = (col + 2 < K) ? src[2] : 0.0f;
+            pf[i].w = (col + 3 < K) ? src[3] : 0.0f;
         }
     };
     // operands of this lane inside the tile: row of token (32 tg + j), columns of pair (2 wave + pl)
@@ -1243,8 +1252,9 @@ int launch_ccs_bf16(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d
                     uint32_t x_cols)
 {
     const uint64_t tiles128 = (uint64_t)((n + 127) / 128) * (g.CB_pad / CcsMfmaShape<V, WIDE>::RCB);
-    // 64-token tiles up to two 128-token tiles per resident workgroup: four workgroups fit a CU instead of three,
-    // and since a workgroup keeps the operands of its codebooks from tile to tile the extra tiles cost little
+    // 64-token tiles up to two 128-token tiles per resident workgroup: the grid fills more evenly, and since a
+    // workgroup keeps the operands of its codebooks from tile to tile the extra tiles cost little (asking the
+    // compiler for four workgroups per CU with them was measured slower: 10.9 against 10.1 us at K = 768)
     // (measured 64 / 128-token tiles, us: 6.1 / 8.7 at 192 tiles; 11.0 / 11.9 at 768; 14.8 / 15.5 at 1188;
     // 17.8 / 18.8 at 1536; 28.2 .. 31.5 / 28.2 .. 29.0 at 3072; 42.3 / 41.8 at 4752)
     const bool small_tiles = g.tune_search_tile ? g.tune_search_tile == 64 : tiles128 <= 6ull * ctx->prop.multiProcessorCount;
