@@ -648,14 +648,21 @@ __global__ __launch_bounds__(CCS_THREADS, 4) void ccs_mfma_kernel(const float* _
 //   cn16  [CB_pad][16] float                   |c|^2 (r for padded codebooks, 3e38 for ids past C)
 // =============================================================================================
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+typedef unsigned int v6u __attribute__((ext_vector_type(6)));
 
 // K-slot registers (two bf16 K-slots each, four registers per MFMA) of lane (row i, half kh).  The lane
-// covers dims DL*kh .. DL*kh + DL-1 (DL = v/2) of both codebooks of the pair; codebook q of the pair owns
-// registers 3*DL*q .. 3*DL*q + 3*DL-1:
-//   DL >= 2: six registers per pair of dims (d, d+1), each (piece of d | piece of d+1 << 16), pieces
-//            {ch, cm, ch, cm, cl, ch} of -2c against the search kernel's {xh, xh, xm, xm, xh, xl};
-//   DL == 1: three registers for the one dim, (ch | cm), (ch | cm), (cl | ch) against (xh | xh), (xm | xm), (xh | xl).
-// Rows of the other codebook, and registers past 6*DL, hold zeros.
+// covers dims DL*kh .. DL*kh + DL-1 (DL = v/2) of both codebooks of the pair.
+//   DL >= 2: three MFMAs per pair of dims (d, d+1); a register holds (piece of d | piece of d+1 << 16).  The
+//            search kernel keeps six registers  xm(cb0) xm(cb1) xh(cb0) xh(cb1) xl(cb0) xl(cb1)  in a row and
+//            hands the MFMAs windows of four of them, so that no piece is copied:
+//              registers 0..3 against {ch, ch, ch, ch}   (xm*ch, xh*ch)
+//              registers 0..3 against {cm, cm, cm, cm}   (xm*cm, xh*cm)
+//              registers 2..5 against {cl, cl, ch, ch}   (xh*cl, xl*ch)
+//            with the pieces of -2c of the row's own codebook in that codebook's registers;
+//   DL == 1: codebook q owns registers 3q .. 3q+2 of the first two MFMAs: (ch | cm), (ch | cm), (cl | ch)
+//            against (xh | xh), (xm | xm), (xh | xl).
+// Registers of the other codebook, and registers past the last one used, hold zeros.
 // WIDE (17..32 centroids): "pair" p is codebook p alone, its half h holds centroids 16h .. 16h+15, and both
 // halves meet the same sub-vector (the search kernel feeds the activations of codebook p to both).
 template <uint32_t V, bool WIDE>
@@ -681,20 +688,18 @@ __global__ void ccs_prep_bf16_kernel(const float* __restrict__ cent, uint4* __re
         pc[d][1] = r1u >> 16;
         pc[d][2] = __float_as_uint(r2) >> 16;
     }
-    const int term[6] = {0, 1, 0, 1, 2, 0};
     for (uint32_t m = 0; m < NM; ++m) {
         uint32_t w[4];
         for (uint32_t q = 0; q < 4; ++q) {
             const uint32_t rho = 4 * m + q;
             uint32_t val = 0;
-            if (real && rho < 6 * DL && rho / (3 * DL) == h) {
-                const uint32_t sg = rho % (3 * DL);
-                if (DL == 1) {
-                    val = sg == 2 ? (pc[0][2] | (pc[0][0] << 16)) : (pc[0][0] | (pc[0][1] << 16));
-                } else {
-                    const uint32_t dp = sg / 6, t = term[sg % 6];
-                    val = pc[2 * dp][t] | (pc[2 * dp + 1][t] << 16);
-                }
+            if (DL == 1) {
+                if (real && rho < 6 && rho / 3 == h)
+                    val = rho % 3 == 2 ? (pc[0][2] | (pc[0][0] << 16)) : (pc[0][0] | (pc[0][1] << 16));
+            } else if (real && (q & 1) == h) {
+                const uint32_t dp = m / 3, kind = m % 3;
+                const uint32_t t = kind == 2 ? (q < 2 ? 2u : 0u) : kind;  // ch, cm, or cl | ch
+                val = pc[2 * dp][t] | (pc[2 * dp + 1][t] << 16);
             }
             w[q] = val;
         }
@@ -871,52 +876,58 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
                     cn_pl[4 * q4 + 3] = c4.w;
                 }
             }
-            uint32_t breg[NM * 4];
-#pragma unroll
-            for (int i = 0; i < NM * 4; ++i) breg[i] = 0;
+            // bf16 pieces of the lane's activations: x = xh + xm + xl exactly
+            uint32_t xu[2][DL], r1u[2][DL], r2u[2][DL];
             float part[2];
 #pragma unroll
             for (int cbh = 0; cbh < 2; ++cbh) {
-                uint32_t xu[DL], r1u[DL], r2u[DL];
                 float sq = 0.0f;
 #pragma unroll
                 for (int d = 0; d < DL; ++d) {
                     const float a = xs[cbh][d];
-                    xu[d] = __float_as_uint(a);
-                    const float r1 = a - __uint_as_float(xu[d] & 0xffff0000u);
-                    r1u[d] = __float_as_uint(r1);
-                    r2u[d] = __float_as_uint(r1 - __uint_as_float(r1u[d] & 0xffff0000u));
+                    xu[cbh][d] = __float_as_uint(a);
+                    const float r1 = a - __uint_as_float(xu[cbh][d] & 0xffff0000u);
+                    r1u[cbh][d] = __float_as_uint(r1);
+                    r2u[cbh][d] = __float_as_uint(r1 - __uint_as_float(r1u[cbh][d] & 0xffff0000u));
                     sq = d == 0 ? a * a : fmaf(a, a, sq);
                 }
                 part[cbh] = sq;
-                // __builtin_amdgcn_perm(p, q, 0x07060302) = (bf16 of q | bf16 of p << 16)
-                if constexpr (DL == 1) {
-                    breg[3 * cbh + 0] = __builtin_amdgcn_perm(xu[0], xu[0], 0x07060302u);    // (xh | xh)
-                    breg[3 * cbh + 1] = __builtin_amdgcn_perm(r1u[0], r1u[0], 0x07060302u);  // (xm | xm)
-                    breg[3 * cbh + 2] = __builtin_amdgcn_perm(r2u[0], xu[0], 0x07060302u);   // (xh | xl)
-                } else {
-#pragma unroll
-                    for (int dp = 0; dp < DL / 2; ++dp) {
-                        const uint32_t H = __builtin_amdgcn_perm(xu[2 * dp + 1], xu[2 * dp], 0x07060302u);
-                        const uint32_t Mm = __builtin_amdgcn_perm(r1u[2 * dp + 1], r1u[2 * dp], 0x07060302u);
-                        const uint32_t L = __builtin_amdgcn_perm(r2u[2 * dp + 1], r2u[2 * dp], 0x07060302u);
-                        const int r0 = 3 * DL * cbh + 6 * dp;
-                        breg[r0 + 0] = H;
-                        breg[r0 + 1] = H;
-                        breg[r0 + 2] = Mm;
-                        breg[r0 + 3] = Mm;
-                        breg[r0 + 4] = H;
-                        breg[r0 + 5] = L;
-                    }
-                }
             }
             // |x|^2 of codebook h: lanes l and l+32 each hold half of it for both codebooks
             const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(part[0]), __float_as_uint(part[1]), false, false);
             xx_out = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+            auto mfma = [&](int m, const v4u& b, bool first) {
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, aq[pl][m]), __builtin_bit_cast(bf16x8, b),
+                                                              first ? cn_pl : acc, 0, 0, 0);
+            };
+            // __builtin_amdgcn_perm(p, q, 0x07060302) = (bf16 of q | bf16 of p << 16)
+            if constexpr (DL == 1) {
+                uint32_t breg[8];
 #pragma unroll
-            for (int m = 0; m < NM; ++m) {
-                const uint4 bm = make_uint4(breg[4 * m], breg[4 * m + 1], breg[4 * m + 2], breg[4 * m + 3]);
-                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, aq[pl][m]), __builtin_bit_cast(bf16x8, bm), m == 0 ? cn_pl : acc, 0, 0, 0);
+                for (int cbh = 0; cbh < 2; ++cbh) {
+                    breg[3 * cbh + 0] = __builtin_amdgcn_perm(xu[cbh][0], xu[cbh][0], 0x07060302u);    // (xh | xh)
+                    breg[3 * cbh + 1] = __builtin_amdgcn_perm(r1u[cbh][0], r1u[cbh][0], 0x07060302u);  // (xm | xm)
+                    breg[3 * cbh + 2] = __builtin_amdgcn_perm(r2u[cbh][0], xu[cbh][0], 0x07060302u);   // (xh | xl)
+                }
+                breg[6] = breg[7] = 0;
+                mfma(0, v4u{breg[0], breg[1], breg[2], breg[3]}, true);
+                mfma(1, v4u{breg[4], breg[5], breg[6], breg[7]}, false);
+            } else {
+#pragma unroll
+                for (int dp = 0; dp < DL / 2; ++dp) {
+                    // six registers in a row, the MFMAs read windows of four of them (see ccs_prep_bf16_kernel)
+                    v6u s6;
+#pragma unroll
+                    for (int cbh = 0; cbh < 2; ++cbh) {
+                        s6[0 + cbh] = __builtin_amdgcn_perm(r1u[cbh][2 * dp + 1], r1u[cbh][2 * dp], 0x07060302u);  // xm
+                        s6[2 + cbh] = __builtin_amdgcn_perm(xu[cbh][2 * dp + 1], xu[cbh][2 * dp], 0x07060302u);    // xh
+                        s6[4 + cbh] = __builtin_amdgcn_perm(r2u[cbh][2 * dp + 1], r2u[cbh][2 * dp], 0x07060302u);  // xl
+                    }
+                    const v4u lo = __builtin_shufflevector(s6, s6, 0, 1, 2, 3), hi = __builtin_shufflevector(s6, s6, 2, 3, 4, 5);
+                    mfma(3 * dp + 0, lo, dp == 0);
+                    mfma(3 * dp + 1, lo, false);
+                    mfma(3 * dp + 2, hi, false);
+                }
             }
         };
 
