@@ -7,7 +7,7 @@ reference's per-tensor fp32 scale, int32 accumulation, random-init centroids and
 One "step" = one pass of the pair (centroid search + LUT gather for FFN1, then for FFN2) with all
 inputs, LUTs and outputs resident in HBM.  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-model] [--no-sweep] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-model] [--no-large-layer] [--no-sweep] [--no-cpu-baseline]
 """
 import argparse
 import json
@@ -263,6 +263,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--tokens", type=int, default=8192)
     ap.add_argument("--no-model", action="store_true", help="skip the 12-layer model forward timing")
+    ap.add_argument("--no-large-layer", action="store_true", help="skip the BERT-large layer timing")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-sweep", action="store_true", help="skip the ViT-Base sweep and the per-codebook-scale pair")
     args = ap.parse_args()
@@ -421,7 +422,8 @@ def main():
                               "note": "pageable host memory in and out of both AMMs (PCIe copies included), 3 steps"}
     if not args.no_model:
         result["bert_base_forward"] = model_forward(pimdl, ctx)
-        result["bert_large_layer"] = bert_large_layer(pimdl, ctx)
+        if not args.no_large_layer:
+            result["bert_large_layer"] = bert_large_layer(pimdl, ctx)
     if not args.no_sweep:
         result["per_codebook_scale"] = per_codebook_scale(pimdl, ctx, rng, N, shapes)
         result["vit_base_sweep"] = vit_sweep(pimdl, ctx)

@@ -1193,13 +1193,13 @@ bool gather_dense_only()
 bool apply_runtime_tuning(AmmGeom* g, const pimdl_amm_tuning& t, std::string* why)
 {
     const bool matrix_core = g->gather_kind != 0;
-    const bool eight_waves = t.token_item == 512 && g->gather_kind == 2;  // one workgroup of eight waves per CU
+    const bool eight_waves = t.token_item == 512 && g->gather_kind == 2 && g->C_tile != 32;  // one workgroup of eight waves per CU
     if (t.token_item && (!matrix_core || (t.token_item != 128 && t.token_item != 256 && !eight_waves))) {
-        *why = "token_item must be 128 or 256 (512 for the sparse kernel), and only the matrix-core gathers (int8, up to 16 centroids) have it";
+        *why = "token_item must be 128 or 256 (512 for the sparse kernel up to 16 centroids), and only the matrix-core gathers (int8, up to 32 centroids) have it";
         return false;
     }
     if (t.cb_per_slice) {
-        const uint32_t entries = g->C_tile == 8 ? g->CB_pad / 2 : g->CB_pad;  // codebooks, or pairs of them
+        const uint32_t entries = g->C_tile == 8 ? g->CB_pad / 2 : g->C_tile == 32 ? 2 * g->CB_pad : g->CB_pad;  // table entries of 16 slots
         const bool has32 = eight_waves || (g->gather_kind == 2 ? g->q <= 4 : (g->q == 3 || (g->q == 4 && g->C_tile != 8)));
         const bool has64 = eight_waves && g->q == 3;
         if (!matrix_core || (t.cb_per_slice == 16 && eight_waves && g->q == 3) ||
@@ -1259,6 +1259,8 @@ bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::s
     g->q = ct >= 128 ? 2 : 4;
     g->gather_kind = (i8 && C <= 16 && !gather_rows_only()) ? 1 : 0;
     if (g->gather_kind == 1 && C > 8 && !gather_dense_only()) g->gather_kind = 2;
+    // 17..32 centroids: the sparse kernel with every codebook as two of 16
+    if (i8 && C > 16 && C <= 32 && !gather_rows_only() && !gather_dense_only()) g->gather_kind = 2;
     switch (tune.gather_kernel) {
         case PIMDL_GATHER_AUTO: break;
         case PIMDL_GATHER_ROWS:
@@ -1269,7 +1271,7 @@ bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::s
             g->gather_kind = 1;
             break;
         case PIMDL_GATHER_SPARSE:
-            if (!(i8 && C > 8 && C <= 16)) { *why = "the sparse one-hot gather needs an int8 table with 9 to 16 centroids"; return false; }
+            if (!(i8 && C > 8 && C <= 32)) { *why = "the sparse one-hot gather needs an int8 table with 9 to 32 centroids"; return false; }
             g->gather_kind = 2;
             break;
         default: *why = "unknown gather_kernel"; return false;
@@ -1282,7 +1284,7 @@ bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::s
         // up to 8 centroids: two codebooks share a lane's 16 K-slots (C_tile 8); 96-column tiles then do not
         // leave room for two workgroups per CU
         const bool paired = C <= 8;
-        g->C_tile = paired ? 8 : 16;
+        g->C_tile = paired ? 8 : C > 16 ? 32 : 16;
         const uint32_t slots = 2 * (num_cus ? num_cus : 256);
         const uint32_t tiles = (d.max_n + 255) / 256;
         double best = 1e300;
@@ -1311,7 +1313,7 @@ bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::s
         g->gather_threads = 256;
         g->tokens_per_wg = 256;
         g->row_pitch = 16;
-        g->gather_lds_bytes = g->gather_kind == 2 ? sparse_lds_bytes(g->q) : (uint32_t)oh_lds_bytes((int)g->q, paired);
+        g->gather_lds_bytes = g->gather_kind == 2 ? sparse_lds_bytes(g->q, C > 16) : (uint32_t)oh_lds_bytes((int)g->q, paired);
         g->M_pad = (M + g->col_block - 1) / g->col_block * g->col_block;
         g->ccs_cb_per_wg = ccs_cb_per_wg(v);
         g->ccs_row_floats = g->ccs_cb_per_wg * v;

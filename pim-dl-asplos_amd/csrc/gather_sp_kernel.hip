@@ -1,4 +1,4 @@
-// LUT gather-accumulate on the sparse matrix instruction (gfx950), int8 tables with 9..16 centroids.
+// LUT gather-accumulate on the sparse matrix instruction (gfx950), int8 tables with 9..32 centroids.
 //
 // Same operator as the other gather kernels (inference-engine/src/dpu/pim_lut_kernel.c:97-2296, row-major
 // statement inference-engine/test/test_amm.cpp:164-175, epilogue inference-engine/src/host/pim_lut_host.cpp:190-203):
@@ -33,6 +33,13 @@
 //
 // Work decomposition, staging through LDS with global_load_lds, the dealing of items to the XCDs, the fused
 // de-quantisation / bias / GELU epilogue and operator groups are those of the dense one-hot kernel.
+//
+// 17..32 centroids (WIDE): a codebook of 32 centroids is two of 16 side by side, of which the token's centroid
+// lies in one and the other contributes nothing.  The table is tiled as 2 CB codebooks of 16 (centroids 0..15,
+// then 16..31), the index row holds one byte per codebook where the 16-centroid form holds two nibbles, and the
+// lane looks its byte up in two 32-entry tables: the first has the one-hot entries for bytes 0..15 and zero
+// entries for 16..31, the second the other way round.  Everything else is the same kernel; one instruction then
+// covers 4 codebooks.
 #include "gather_common.h"
 
 namespace pimdl {
@@ -58,10 +65,10 @@ typedef int v2i __attribute__((ext_vector_type(2)));
 // to one workgroup (slices twice as deep, half as many barriers).
 constexpr int sp_tok_item(int tm, int nw = 4) { return nw * tm * 16; }
 constexpr int sp_nbuf(int gs) { return gs > 16 ? 2 : 3; }
-constexpr int SP_TABLE = 256;  // 16 entries of 16 bytes
-constexpr int sp_lds_bytes(int tn, int gs, int nw = 4)
+constexpr int sp_table_bytes(bool wide) { return wide ? 1024 : 256; }  // 16 entries of 16 bytes, or two tables of 32
+constexpr int sp_lds_bytes(int tn, int gs, int nw = 4, bool wide = false)
 {
-    return SP_TABLE + sp_nbuf(gs) * gs * 16 * tn * 16 + sp_nbuf(gs) * nw * 64 * 4 * (gs / 8);
+    return sp_table_bytes(wide) + sp_nbuf(gs) * gs * 16 * tn * 16 + sp_nbuf(gs) * nw * 64 * 4 * (gs / 8);
 }
 
 template <int OFF>
@@ -84,7 +91,8 @@ __device__ __forceinline__ T* uniform_ptr(T* p)
     return reinterpret_cast<T*>(((uint64_t)hi << 32) | lo);
 }
 
-template <int TN, int TM, int GS, int NW>
+// CB_pad: codebooks of 16 centroids in the tiled table (twice the operator's for WIDE)
+template <int TN, int TM, int GS, int NW, bool WIDE>
 __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel(
     const uint8_t* __restrict__ idx, const int8_t* __restrict__ lut, float* __restrict__ out,
     int32_t* __restrict__ acc_out, uint32_t N, uint32_t M, uint32_t CB_pad, uint32_t idx_row_bytes,
@@ -106,7 +114,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     constexpr int NBUF = sp_nbuf(GS), NIBUF = NBUF;
     constexpr int PD = NBUF - 1;  // prefetch distance of the LUT stream, in slices
-    constexpr uint32_t BUF0 = SP_TABLE;
+    constexpr uint32_t BUF0 = sp_table_bytes(WIDE);
     constexpr uint32_t IBUF0 = BUF0 + NBUF * SLICE;
     constexpr uint32_t IBYTES = SP_WAVES * 64 * 4 * IWORDS;   // index bytes of one slice (a 64-token block per wave)
     constexpr uint32_t IWAVE = 64 * 4 * IWORDS;               // ... of one wave's 64 tokens
@@ -125,11 +133,15 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel
     // Table entry c (16 bytes): value bytes of a codebook whose centroid is c (first slot of group c / 4 is 1),
     // then the position bits (c % 4 at value slot 2 (c / 4), two bits per slot) as they stand in the low half
     // of the lane's position word, then the same bits shifted to the high half.
-    if (threadIdx.x < 64) {
-        const uint32_t c = threadIdx.x >> 2, w = threadIdx.x & 3, grp = c >> 2, pos = c & 3;
+    // WIDE: table h (h = 0, 1; 512 bytes each) has entry c at byte b = 16 h + c and zero entries elsewhere.
+    static_assert(NW * 64 >= 256, "one table word per thread");
+    if (threadIdx.x < (WIDE ? 256 : 64)) {
+        const uint32_t b = (threadIdx.x >> 2) & 31, table = threadIdx.x >> 7;
+        const uint32_t c = b & 15, w = threadIdx.x & 3, grp = c >> 2, pos = c & 3;
         uint32_t word;
         if (w < 2) word = (grp >> 1) == w ? (1u << (16 * (grp & 1))) : 0u;  // value bytes 0..3 / 4..7: slot 2 grp
         else word = (pos << (4 * grp)) << (w == 3 ? 16 : 0);
+        if (WIDE && (b >> 4) != table) word = 0;
         reinterpret_cast<uint32_t*>(smem)[threadIdx.x] = word;
     }
 
@@ -232,8 +244,13 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel
         for (int t = 0; t < TM; ++t)
 #pragma unroll
             for (int i = 0; i < IWORDS; ++i) {
-                lo[t][i] = (raw[t][i] << 4) & 0xF0u;
-                hi[t][i] = raw[t][i] & 0xF0u;
+                if constexpr (WIDE) {  // the byte is one codebook's centroid: its entry in the first and in the second table
+                    lo[t][i] = raw[t][i] << 4;
+                    hi[t][i] = lo[t][i] + 512;
+                } else {
+                    lo[t][i] = (raw[t][i] << 4) & 0xF0u;
+                    hi[t][i] = raw[t][i] & 0xF0u;
+                }
             }
     };
 
@@ -438,14 +455,15 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel
     }
 }
 
-template <int TN, int TM, int GS, int NW = 4>
+template <int TN, int TM, int GS, int NW = 4, bool WIDE = false>
 int launch_sparse_tm(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_t* d_acc, uint32_t n,
                      const Epilogue& ep)
 {
-    constexpr int LDS = sp_lds_bytes(TN, GS, NW);
+    constexpr int LDS = sp_lds_bytes(TN, GS, NW, WIDE);
     static_assert((NW == 4 ? 2 : 1) * LDS <= 160 * 1024, "two workgroups of four waves, or one of eight, per CU");
     constexpr int TOK_ITEM = sp_tok_item(TM, NW);
-    auto kern = gather_sparse_kernel<TN, TM, GS, NW>;
+    auto kern = gather_sparse_kernel<TN, TM, GS, NW, WIDE>;
+    const uint32_t cb16 = sparse_codebooks(a.g);  // codebooks of 16 centroids in the tiled table
     static bool attr_set = false;
     if (!attr_set) {
         int rc = hip_check(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -458,19 +476,20 @@ int launch_sparse_tm(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out,
     const uint32_t n_items = n_token_tiles * (a.g.M_pad / (16 * TN));
     uint32_t grid = ctx->prop.multiProcessorCount * (NW == 4 ? 2 : 1);
     if (grid > n_items) grid = n_items;
-    const XcdMap xmap = choose_xcd_map(a.g.M_pad / (16 * TN), n_token_tiles, grid, (uint64_t)a.g.CB_pad * 16 * a.g.M_pad,
+    const XcdMap xmap = choose_xcd_map(a.g.M_pad / (16 * TN), n_token_tiles, grid, (uint64_t)cb16 * 16 * a.g.M_pad,
                                        (uint64_t)n * a.g.idx_row_bytes, a.g.tune_xcd_col_split);
-    snprintf(a.last_gather, sizeof(a.last_gather), "gather_sparse_kernel<%d, %d, %d, %d>", TN, TM, GS, NW);
+    snprintf(a.last_gather, sizeof(a.last_gather), "gather_sparse_kernel<%d, %d, %d, %d, %s>", TN, TM, GS, NW, WIDE ? "true" : "false");
     a.note_launch(GS, LDS, TOK_ITEM, NW * 64);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), LDS, ctx->stream, d_idx, reinterpret_cast<const int8_t*>(a.d_lut),
-                       d_out, d_acc, n, a.g.M, a.g.CB_pad, a.g.idx_row_bytes, n_token_tiles, n_items, ep, xmap);
+                       d_out, d_acc, n, a.g.M, cb16, a.g.idx_row_bytes, n_token_tiles, n_items, ep, xmap);
     return hip_check(ctx, hipGetLastError(), "gather_sparse_kernel launch");
 }
 
 // 256- or 128-token items, whichever gives the shorter launch (the rule of the dense kernel)
-template <int TN>
+template <int TN, bool WIDE>
 int launch_sparse_tn(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_t* d_acc, uint32_t n, const Epilogue& ep)
 {
+    const uint32_t cb16 = sparse_codebooks(a.g);
     const uint64_t col_tiles = a.g.M_pad / (16 * TN);
     const uint64_t items4 = (uint64_t)((n + sp_tok_item(4) - 1) / sp_tok_item(4)) * col_tiles;
     const uint64_t items2 = (uint64_t)((n + sp_tok_item(2) - 1) / sp_tok_item(2)) * col_tiles;
@@ -482,16 +501,16 @@ int launch_sparse_tn(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out,
     // and can be 64 codebooks deep (measured 44.1 -> 42.4 us at 3072 -> 768, N = 8192; the 96-column kernel
     // loses 3 us the same way, its two waves of a SIMD then waiting at the same barrier).  Taken where it costs
     // no extra round of the grid and still gives every CU a workgroup.
-    if constexpr (TN == 3) {
+    if constexpr (TN == 3 && !WIDE) {
         const uint64_t cus = ctx->prop.multiProcessorCount;
         const uint64_t items8 = (uint64_t)((n + sp_tok_item(4, 8) - 1) / sp_tok_item(4, 8)) * col_tiles;
-        if (!a.g.tune_token_item && !a.g.tune_cb_per_slice && a.g.CB_pad % 64 == 0 && !small_items && items8 >= cus &&
+        if (!a.g.tune_token_item && !a.g.tune_cb_per_slice && cb16 % 64 == 0 && !small_items && items8 >= cus &&
             (items8 + cus - 1) / cus <= (items4 + slots - 1) / slots)
             return launch_sparse_tm<TN, 4, 64, 8>(ctx, a, d_idx, d_out, d_acc, n, ep);
     }
-    if (a.g.tune_token_item == 512) {  // one workgroup of eight waves per CU
+    if constexpr (!WIDE) if (a.g.tune_token_item == 512) {  // one workgroup of eight waves per CU
         if constexpr (TN == 3) {
-            if (a.g.CB_pad % 64 == 0 && a.g.tune_cb_per_slice == 64) return launch_sparse_tm<TN, 4, 64, 8>(ctx, a, d_idx, d_out, d_acc, n, ep);
+            if (cb16 % 64 == 0 && a.g.tune_cb_per_slice == 64) return launch_sparse_tm<TN, 4, 64, 8>(ctx, a, d_idx, d_out, d_acc, n, ep);
         }
         // (CB_pad is a multiple of 32; 48-column tiles have no 16-codebook variant here: 12 blocks for 8 waves)
         if (TN == 3 || a.g.tune_cb_per_slice != 16) return launch_sparse_tm<TN, 4, 32, 8>(ctx, a, d_idx, d_out, d_acc, n, ep);
@@ -499,18 +518,18 @@ int launch_sparse_tn(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out,
     }
     constexpr int GSB = TN <= 4 ? 32 : 16;  // 32-codebook slices in two buffers where two workgroups still fit a CU
     if constexpr (GSB != 16) {
-        if (a.g.CB_pad % GSB == 0 && a.g.tune_cb_per_slice != 16) {
-            if (small_items) return launch_sparse_tm<TN, 2, GSB>(ctx, a, d_idx, d_out, d_acc, n, ep);
-            return launch_sparse_tm<TN, 4, GSB>(ctx, a, d_idx, d_out, d_acc, n, ep);
+        if (cb16 % GSB == 0 && a.g.tune_cb_per_slice != 16) {
+            if (small_items) return launch_sparse_tm<TN, 2, GSB, 4, WIDE>(ctx, a, d_idx, d_out, d_acc, n, ep);
+            return launch_sparse_tm<TN, 4, GSB, 4, WIDE>(ctx, a, d_idx, d_out, d_acc, n, ep);
         }
     }
-    if (small_items) return launch_sparse_tm<TN, 2, 16>(ctx, a, d_idx, d_out, d_acc, n, ep);
-    return launch_sparse_tm<TN, 4, 16>(ctx, a, d_idx, d_out, d_acc, n, ep);
+    if (small_items) return launch_sparse_tm<TN, 2, 16, 4, WIDE>(ctx, a, d_idx, d_out, d_acc, n, ep);
+    return launch_sparse_tm<TN, 4, 16, 4, WIDE>(ctx, a, d_idx, d_out, d_acc, n, ep);
 }
 
 }  // namespace
 
-uint32_t sparse_lds_bytes(uint32_t tn) { return (uint32_t)sp_lds_bytes((int)tn, 16); }
+uint32_t sparse_lds_bytes(uint32_t tn, bool wide) { return (uint32_t)sp_lds_bytes((int)tn, 16, 4, wide); }
 
 int launch_gather_sparse(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_t* d_acc, uint32_t n,
                          float scale, float lut_bias_term)
@@ -523,10 +542,18 @@ int launch_gather_sparse(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_
     ep.op_scales = a.d_op_scales;
     ep.op_col_tiles = a.op_col_tiles;
     ep.op_idx_stride = a.op_idx_stride;
-    switch (a.g.q) {
-        case 3: return launch_sparse_tn<3>(ctx, a, d_idx, d_out, d_acc, n, ep);
-        case 4: return launch_sparse_tn<4>(ctx, a, d_idx, d_out, d_acc, n, ep);
-        case 6: return launch_sparse_tn<6>(ctx, a, d_idx, d_out, d_acc, n, ep);
+    if (a.g.C_tile == 32) {
+        switch (a.g.q) {
+            case 3: return launch_sparse_tn<3, true>(ctx, a, d_idx, d_out, d_acc, n, ep);
+            case 4: return launch_sparse_tn<4, true>(ctx, a, d_idx, d_out, d_acc, n, ep);
+            case 6: return launch_sparse_tn<6, true>(ctx, a, d_idx, d_out, d_acc, n, ep);
+        }
+    } else {
+        switch (a.g.q) {
+            case 3: return launch_sparse_tn<3, false>(ctx, a, d_idx, d_out, d_acc, n, ep);
+            case 4: return launch_sparse_tn<4, false>(ctx, a, d_idx, d_out, d_acc, n, ep);
+            case 6: return launch_sparse_tn<6, false>(ctx, a, d_idx, d_out, d_acc, n, ep);
+        }
     }
     return set_error(ctx, PIMDL_ERR_UNSUPPORTED, "no sparse gather kernel for %u column groups", a.g.q);
 }

@@ -184,7 +184,7 @@ static void retile_lut(const T* lut, T* tiled, const AmmGeom& g, uint32_t row_el
 static void retile_lut_onehot(const int8_t* lut, int8_t* tiled, const AmmGeom& g)
 {
     const uint32_t wn = g.col_block;
-    const bool paired = g.C_tile == 8;
+    const bool paired = g.C_tile == 8, wide = g.C_tile == 32;
     // position of column f % wn inside its tile: the sparse-instruction kernel deals a tile's columns to its
     // 16-column groups so that a lane's accumulators are consecutive columns
     std::vector<uint32_t> where(wn);
@@ -192,8 +192,10 @@ static void retile_lut_onehot(const int8_t* lut, int8_t* tiled, const AmmGeom& g
     for (uint32_t cb = 0; cb < g.CB; ++cb)
         for (uint32_t c = 0; c < g.C; ++c) {
             const int8_t* src = lut + ((size_t)cb * g.C + c) * g.M;
-            const uint32_t entry = paired ? cb / 2 : cb, entries = paired ? g.CB_pad / 2 : g.CB_pad;
-            const uint32_t slot = paired ? 8 * (cb & 1) + c : c;
+            // an entry is 16 slots: a codebook; two codebooks of up to 8 centroids; half a codebook of 17..32
+            const uint32_t entry = paired ? cb / 2 : wide ? 2 * cb + c / 16 : cb;
+            const uint32_t entries = paired ? g.CB_pad / 2 : wide ? 2 * g.CB_pad : g.CB_pad;
+            const uint32_t slot = paired ? 8 * (cb & 1) + c : c % 16;
             for (uint32_t f = 0; f < g.M; ++f)
                 tiled[((((size_t)(f / wn) * entries + entry) * wn) + where[f % wn]) * 16 + slot] = src[f];
         }

@@ -161,7 +161,9 @@ int launch_diag_mfma_error(Ctx* ctx, uint32_t trials, bool crafted, float* max_e
 int launch_gather_sparse(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_t* d_acc_or_null,
                          uint32_t n, float scale, float lut_bias_term);
 uint32_t sparse_tile_column(uint32_t tn, uint32_t s);  // column of a tile stored at position s of the tile
-uint32_t sparse_lds_bytes(uint32_t tn);
+uint32_t sparse_lds_bytes(uint32_t tn, bool wide);
+// codebooks of 16 centroids in the table of the sparse one-hot gather: a codebook of 17..32 centroids is two
+inline uint32_t sparse_codebooks(const AmmGeom& g) { return g.C_tile == 32 ? 2 * g.CB_pad : g.CB_pad; }
 bool gather_dense_only();
 
 uint32_t ccs_cb_per_wg(uint32_t v);  // codebooks one ccs workgroup covers (0: generic kernel)

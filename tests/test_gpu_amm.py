@@ -199,9 +199,10 @@ def test_near_ties_follow_the_scan_not_the_true_argmin(ctx):
     amm.close()
 
 
-@pytest.mark.parametrize("C", [16, 8, 5])
+@pytest.mark.parametrize("C", [16, 8, 5, 32, 20, 64])
 def test_gather_from_given_indices_and_invariants(ctx, C):
-    """C <= 8 runs the paired form of the matrix-core gather (two codebooks per index byte, odd CB)."""
+    """C <= 8 runs the paired form of the matrix-core gather (two codebooks per index byte, odd CB), 17..32 the
+    sparse form with every codebook as two of 16 (byte indices), more than 32 the byte adder."""
     rng = np.random.default_rng(21)
     N, CB, M, v = 300, 41 if C < 16 else 40, 192, 4
     cent = rng.standard_normal((CB, C, v)).astype(np.float32)
@@ -280,7 +281,8 @@ def test_two_tokens_per_lane_in_the_fp32_table_gather(ctx, kind):
     (1300, 128, 4, 8, (192, 192, 192), "i8"),   # paired gather, three members in one gather launch
     (700, 256, 4, 16, (96, 96), "i8"),          # one gather launch, 96-column tiles
     (2100, 128, 4, 16, (768, 768, 768), "i8"),  # the Q/K/V shape
-    (257, 256, 2, 32, (100, 60), "i8"),         # 32 centroids: byte indices, row-major index rows
+    (257, 256, 2, 32, (100, 60), "i8"),         # 32 centroids: byte indices, tiled index rows (sparse gather, two tables)
+    (900, 256, 4, 32, (96, 96, 96), "i8"),      # 32 centroids, three members in one gather launch
     (300, 256, 8, 16, (48, 80, 48), "f32"),     # fp32 tables
 ])
 def test_operators_sharing_an_input_are_searched_by_one_launch(ctx, N, K, v, C, Ms, lut):
@@ -301,7 +303,7 @@ def test_operators_sharing_an_input_are_searched_by_one_launch(ctx, N, K, v, C, 
     for o, o2 in zip(outs, outs2):
         assert np.array_equal(o[:77], o2)
     # one gather launch for all members where they are matrix-core gathers of one shape
-    same_shape = lut == "i8" and C <= 16 and len(set(Ms)) == 1 and Ms[0] % amms[0].geometry()["col_block"] == 0
+    same_shape = lut == "i8" and C <= 32 and len(set(Ms)) == 1 and Ms[0] % amms[0].geometry()["col_block"] == 0
     assert (group.fused_cols > 0) == same_shape
     if same_shape:
         fused = group.run_fused(x)

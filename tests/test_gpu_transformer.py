@@ -407,14 +407,32 @@ def test_every_tuning_choice_gives_the_same_bits(ctx):
             amm.set_tuning(token_item=100)
         amm.close()
     assert seen > 100
-    # more than 16 centroids: only the byte adder, and no fp32 matrix-core search
+    # 17..32 centroids: the sparse kernel (every codebook as two of 16) or the byte adder; no dense one-hot
+    # kernel, no fp32 matrix-core search, no eight-wave workgroups
     lut32 = rng.integers(-128, 128, (CB, 32, M)).astype(np.int8)
     cent32 = rng.standard_normal((CB, 32, v)).astype(np.float32)
-    for bad in ({"gather_kernel": pimdl.GATHER_SPARSE}, {"gather_kernel": pimdl.GATHER_ONEHOT}, {"search_kernel": 2},
-                {"token_item": 128}):
+    want32, _, _ = oracle.amm_cpu(x, cent32, lut32, bias, v, 0.02, 0.0, threads=8)
+    for bad in ({"gather_kernel": pimdl.GATHER_ONEHOT}, {"search_kernel": 2}, {"token_item": 512},
+                {"gather_kernel": pimdl.GATHER_ROWS, "token_item": 128}):
         with pytest.raises(pimdl.PimdlError) as e:
             ctx.amm(cent32, lut32, np.float32(0.02), None, max_n=N, tuning=bad)
         assert e.value.code == pimdl.ERR_INVALID
+    for gk, cb in ((pimdl.GATHER_ROWS, 48), (pimdl.GATHER_ROWS, 64), (pimdl.GATHER_SPARSE, 48), (pimdl.GATHER_SPARSE, 64),
+                   (pimdl.GATHER_SPARSE, 96)):
+        amm = ctx.amm(cent32, lut32, np.float32(0.02), bias, max_n=N, tuning={"gather_kernel": gk, "col_block": cb})
+        settings = [{}]
+        if gk == pimdl.GATHER_SPARSE:
+            settings += [{"token_item": 128}, {"token_item": 256}, {"cb_per_slice": 16}, {"xcd_col_split": 2}]
+            if cb <= 64:
+                settings.append({"cb_per_slice": 32, "token_item": 128})
+        for st in settings:
+            amm.set_tuning(**st)
+            assert np.array_equal(amm.run(x).view(np.uint32), want32.view(np.uint32)), (gk, cb, st)
+        assert amm.last_gather_kernel().startswith("gather_sparse" if gk == pimdl.GATHER_SPARSE else "gather_i8")
+        amm.close()
+    with pytest.raises(pimdl.PimdlError):   # 33 centroids and more: the byte adder only
+        ctx.amm(rng.standard_normal((CB, 40, v)).astype(np.float32), rng.integers(-128, 128, (CB, 40, M)).astype(np.int8),
+                np.float32(0.02), None, max_n=N, tuning={"gather_kernel": pimdl.GATHER_SPARSE})
 
 
 def test_full_measured_search_runs(ctx):
