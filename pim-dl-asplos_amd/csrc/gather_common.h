@@ -39,9 +39,10 @@ inline double grid_rounds(uint64_t items, uint64_t slots)
 }
 // Time of one item of the matrix-core gathers relative to a 256-token x 96-column one (same number of codebooks):
 // 64- and 48-column tiles read the one-hot operand for fewer column groups (measured per round at 768 -> 3072,
-// N = 8192, launch overhead taken off: 21.5 / 14.7 / 13.1 us; 27.9 / 19.2 at 1024 -> 4096); a 128-token item takes
-// 0.62 of a 256-token one.
-inline double item_cost(uint32_t tn, bool small_item) { return (tn >= 6 ? 1.0 : tn == 4 ? 0.70 : 0.61) * (small_item ? 0.62 : 1.0); }
+// N = 8192, launch overhead taken off: 21.5 / 14.7 / 13.1 us; 27.9 / 19.2 at 1024 -> 4096; the 64-column figure is
+// set a little above the measured 0.68 .. 0.72 so that near ties go to the wider tile, which won them: 768 -> 3072
+// at N = 12608 with 32 centroids, 131.8 against 139.3 us); a 128-token item takes 0.62 of a 256-token one.
+inline double item_cost(uint32_t tn, bool small_item) { return (tn >= 6 ? 1.0 : tn == 4 ? 0.72 : 0.61) * (small_item ? 0.62 : 1.0); }
 // 128-token items instead of 256-token ones where that is the shorter launch by the two figures above.
 inline bool prefer_small_items(uint64_t items256, uint64_t items128, uint64_t slots)
 {
