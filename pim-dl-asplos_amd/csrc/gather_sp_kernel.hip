@@ -499,13 +499,16 @@ int launch_sparse_tn(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out,
     // 48-column tiles read the sparse operand of a token group for three column groups only, so the copies and
     // the per-slice costs weigh most there: with eight waves per workgroup a slice is copied once per 512 tokens
     // and can be 64 codebooks deep (measured 44.1 -> 42.4 us at 3072 -> 768, N = 8192; the 96-column kernel
-    // loses 3 us the same way, its two waves of a SIMD then waiting at the same barrier).  Taken where it costs
-    // no extra round of the grid and still gives every CU a workgroup.
+    // loses 3 us the same way, its two waves of a SIMD then waiting at the same barrier).  Taken where it gives the
+    // shorter launch: a round of 512-token items takes 0.96 of a round of twice as many 256-token items, but a partly
+    // filled last round costs a whole one (its workgroups are alone on their CUs either way), where four-wave
+    // workgroups speed up (grid_rounds): the fused Q/K/V gather at N = 4096 (1.5 rounds) takes 21.7 us with four
+    // waves and 27.4 us with eight.
     if constexpr (TN == 3 && !WIDE) {
         const uint64_t cus = ctx->prop.multiProcessorCount;
         const uint64_t items8 = (uint64_t)((n + sp_tok_item(4, 8) - 1) / sp_tok_item(4, 8)) * col_tiles;
         if (!a.g.tune_token_item && !a.g.tune_cb_per_slice && cb16 % 64 == 0 && !small_items && items8 >= cus &&
-            (items8 + cus - 1) / cus <= (items4 + slots - 1) / slots)
+            0.96 * (double)((items8 + cus - 1) / cus) < grid_rounds(items4, slots))
             return launch_sparse_tm<TN, 4, 64, 8>(ctx, a, d_idx, d_out, d_acc, n, ep);
     }
     if constexpr (!WIDE) if (a.g.tune_token_item == 512) {  // one workgroup of eight waves per CU
