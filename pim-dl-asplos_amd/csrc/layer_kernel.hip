@@ -145,7 +145,7 @@ __global__ __launch_bounds__(256) void layer_norm_vec_kernel(const float* __rest
 constexpr int AT_KC = 128, AT_PITCH = 68, AT_THREADS = 256;
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-__global__ __launch_bounds__(AT_THREADS) void attention_hd64_kernel(const float* __restrict__ q,
+__global__ __launch_bounds__(AT_THREADS, 3) void attention_hd64_kernel(const float* __restrict__ q,
                                                                    const float* __restrict__ k,
                                                                    const float* __restrict__ v,
                                                                    float* __restrict__ out, uint32_t S,
@@ -172,14 +172,25 @@ __global__ __launch_bounds__(AT_THREADS) void attention_hd64_kernel(const float*
             qreg[4 * i + 3] = t.w * scale;
         }
     }
-    auto load_chunk = [&](const float* src, uint32_t kc) {  // 128 keys x 64 floats -> LDS, zero past S
-        for (uint32_t i = threadIdx.x; i < AT_KC * 16; i += AT_THREADS) {
-            const uint32_t key = i / 16, c4 = i % 16, tok = kc + key;
-            float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (tok < S) t = *reinterpret_cast<const float4*>(src + in_base + (size_t)tok * in_stride + 4 * c4);
-            *reinterpret_cast<float4*>(&kv[key * AT_PITCH + 4 * c4]) = t;
+    // 128 keys x 64 floats, zero past S: into registers (eight 16-byte pieces per thread), then into LDS.  The two
+    // halves are separate so that V is already on its way while the scores are computed from K.
+    constexpr int AT_PIECES = AT_KC * 16 / AT_THREADS;
+    auto fetch_chunk = [&](float4 (&r)[AT_PIECES], const float* src, uint32_t kc) {
+#pragma unroll
+        for (int p = 0; p < AT_PIECES; ++p) {
+            const uint32_t i = threadIdx.x + p * AT_THREADS, key = i / 16, c4 = i % 16, tok = kc + key;
+            r[p] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (tok < S) r[p] = *reinterpret_cast<const float4*>(src + in_base + (size_t)tok * in_stride + 4 * c4);
         }
     };
+    auto store_chunk = [&](const float4 (&r)[AT_PIECES]) {
+#pragma unroll
+        for (int p = 0; p < AT_PIECES; ++p) {
+            const uint32_t i = threadIdx.x + p * AT_THREADS, key = i / 16, c4 = i % 16;
+            *reinterpret_cast<float4*>(&kv[key * AT_PITCH + 4 * c4]) = r[p];
+        }
+    };
+    float4 stage[AT_PIECES];
 
     float m_run = -__builtin_inff(), l_run = 0.0f;
     v4f o[4];
@@ -187,12 +198,18 @@ __global__ __launch_bounds__(AT_THREADS) void attention_hd64_kernel(const float*
     for (int dt = 0; dt < 4; ++dt) o[dt] = (v4f){0.f, 0.f, 0.f, 0.f};
 
     for (uint32_t kc = 0; kc < S; kc += AT_KC) {
+        fetch_chunk(stage, k, kc);
         __syncthreads();  // the previous chunk's V has been consumed
-        load_chunk(k, kc);
+        store_chunk(stage);
         __syncthreads();
+        fetch_chunk(stage, v, kc);  // lands while the scores are computed
         v4f s[AT_KC / 16];
 #pragma unroll
         for (int kt = 0; kt < AT_KC / 16; ++kt) {
+            if (kc + 16 * kt >= S) {  // (uniform) a key tile past the sequence: nothing to compute
+                s[kt] = (v4f){0.f, 0.f, 0.f, 0.f};
+                continue;
+            }
             const float* kp = kv + (16 * kt + j) * AT_PITCH + 16 * g;
             float areg[16];
 #pragma unroll
@@ -238,10 +255,11 @@ __global__ __launch_bounds__(AT_THREADS) void attention_hd64_kernel(const float*
         for (int dt = 0; dt < 4; ++dt) o[dt] *= alpha;
 
         __syncthreads();  // every wave is done with K
-        load_chunk(v, kc);
+        store_chunk(stage);
         __syncthreads();
 #pragma unroll
-        for (int kt = 0; kt < AT_KC / 16; ++kt)
+        for (int kt = 0; kt < AT_KC / 16; ++kt) {
+            if (kc + 16 * kt >= S) continue;  // (uniform) its probabilities are all zero
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const float* vp = kv + (16 * kt + 4 * g + i) * AT_PITCH + j;
@@ -249,6 +267,7 @@ __global__ __launch_bounds__(AT_THREADS) void attention_hd64_kernel(const float*
                 for (int dt = 0; dt < 4; ++dt)
                     o[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(vp[16 * dt], s[kt][i], o[dt], 0, 0, 0);
             }
+        }
     }
     if (q_tok < S) {
         const float inv = 1.0f / l_run;
