@@ -129,8 +129,9 @@ __global__ __launch_bounds__(256) void layer_norm_vec_kernel(const float* __rest
 // output stay in the layer's [token][head * 64 + d] order, so no head transposes are needed.
 //
 // A workgroup = 64 queries of one (batch, head), a wave = 16 of them.  Keys come in chunks of 128
-// through LDS (K, then V in the same buffer), with the running maximum / sum of a streaming softmax
-// between chunks.  Both products run on v_mfma_f32_16x16x4_f32, transposed so that nothing has to
+// through LDS (K, then V in the same buffer; V is fetched into registers while the scores are computed from
+// K), with the running maximum / sum of a streaming softmax between chunks; 16-key tiles past the end of
+// the sequence are skipped.  Both products run on v_mfma_f32_16x16x4_f32, transposed so that nothing has to
 // change lanes in between:
 //   S^T[key][query]  = K Q^T:  A = K rows (keys), B = this lane's query, 16 steps of 4 dims.  The K
 //                      index of lane group g in step s is dim 16 g + s (a sum does not care in which
