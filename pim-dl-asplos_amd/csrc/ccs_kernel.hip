@@ -294,7 +294,7 @@ __global__ __launch_bounds__(CCS_THREADS) void ccs_kernel(const float* __restric
             const float* __restrict__ cp = cent + (size_t)cb * C * V;
             float best = 0.0f;
             bi = 0;
-#pragma unroll 4
+#pragma unroll 8
             for (uint32_t c = 0; c < C; ++c) {
                 // d = ((0 + d0*d0) + d1*d1) + ... ; 0.0f + p == p exactly for every p >= 0
                 float diff = __fsub_rn(xv[cbl * V + 0], cp[c * V + 0]);
@@ -1019,7 +1019,9 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
                     const float* xo = brow0 + tg * 32 * PITCH + pl * XSTEP + (WIDE ? 0 : V * h);
                     const float* cp = cst + cbl * C * V;
                     float best = 0.0f;
-#pragma nounroll
+                    // eight centroids per trip: their rows are read from LDS together, and the wave waits for
+                    // LDS once per trip instead of once per centroid (rolled, a replay took 1.5 us)
+#pragma unroll 8
                     for (uint32_t c = 0; c < C; ++c) {
                         float diff = __fsub_rn(xo[0], cp[c * V + 0]);
                         float d = __fmul_rn(diff, diff);
