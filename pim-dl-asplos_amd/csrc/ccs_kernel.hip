@@ -294,7 +294,7 @@ __global__ __launch_bounds__(CCS_THREADS) void ccs_kernel(const float* __restric
             const float* __restrict__ cp = cent + (size_t)cb * C * V;
             float best = 0.0f;
             bi = 0;
-#pragma unroll 8
+#pragma unroll 4
             for (uint32_t c = 0; c < C; ++c) {
                 // d = ((0 + d0*d0) + d1*d1) + ... ; 0.0f + p == p exactly for every p >= 0
                 float diff = __fsub_rn(xv[cbl * V + 0], cp[c * V + 0]);
