@@ -1051,7 +1051,10 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
         // ---- merge the two codebooks of each pair (lanes l and l+32), gather the tile's index
         //      bytes in LDS, store 8 bytes per token ------------------------------------------------
 #pragma unroll
-        for (int i = 0; i < TG / 2; ++i) words[i] |= __shfl_xor(words[i], 32);
+        for (int i = 0; i < TG / 2; ++i) {  // lanes l and l + 32 exchange their words without going through LDS
+            const auto sw = __builtin_amdgcn_permlane32_swap(words[i], words[i], false, false);
+            words[i] = sw[0] | sw[1];
+        }
         if (h == 0) {
 #pragma unroll
             for (int tg = 0; tg < TG; ++tg)
