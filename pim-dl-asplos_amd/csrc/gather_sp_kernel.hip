@@ -17,8 +17,9 @@
 //             0..7) and 2g+1 (value bytes 8..15): each codebook is four groups of two value slots; the group
 //             that contains the token's centroid c (group c / 4) has value 1 in its first slot with position
 //             c % 4, everything else is 0.  Both codebooks' nibbles are one byte of the packed index row.
-//             The 8 value bytes and the 16 position bits of a nibble come from a 256-byte table in LDS
-//             (entry c: 8 value bytes, position bits for the low half, position bits for the high half).
+//             The 8 value bytes of a nibble come from a 256-byte table in LDS (entry c, 16 bytes apart: 8-byte
+//             reads of such entries do not meet in a bank), the lane's whole position word (16 bits per nibble)
+//             from a second table with one 4-byte word per value of the index byte.
 //   dense B (K x columns)  lane (g, j) holds column j's 16 centroid entries of codebook g (bytes 0..15) and
 //             of codebook g + 4 (bytes 16..31): two 16-byte reads of the tiled table, whose layout is that
 //             of the dense one-hot kernel ([column tile][codebook][column][16 centroids]).
@@ -65,7 +66,9 @@ typedef int v2i __attribute__((ext_vector_type(2)));
 // to one workgroup (slices twice as deep, half as many barriers).
 constexpr int sp_tok_item(int tm, int nw = 4) { return nw * tm * 16; }
 constexpr int sp_nbuf(int gs) { return gs > 16 ? 2 : 3; }
-constexpr int sp_table_bytes(bool wide) { return wide ? 1024 : 256; }  // 16 entries of 16 bytes, or two tables of 32
+// value table(s): 16 entries of 16 bytes, or two tables of 32; then the position words, one per index byte
+constexpr int sp_value_table_bytes(bool wide) { return wide ? 1024 : 256; }
+constexpr int sp_table_bytes(bool wide) { return sp_value_table_bytes(wide) + 1024; }
 constexpr int sp_lds_bytes(int tn, int gs, int nw = 4, bool wide = false)
 {
     return sp_table_bytes(wide) + sp_nbuf(gs) * gs * 16 * tn * 16 + sp_nbuf(gs) * nw * 64 * 4 * (gs / 8);
@@ -75,6 +78,11 @@ template <int OFF>
 __device__ __forceinline__ void lds_read64(v2i& dst, uint32_t addr)
 {
     asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+template <int OFF>
+__device__ __forceinline__ void lds_read32(int& dst, uint32_t addr)
+{
+    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
 }
 template <int N>
 __device__ __forceinline__ void lgkm_wait()
@@ -110,10 +118,11 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel
     constexpr int DMA_PER_WAVE = (NBLK + SP_WAVES - 1) / SP_WAVES;
     static_assert(KSTEPS >= 2, "the operand pipeline below re-arms inside a slice");
 
-    // LDS: table (256 B) | NBUF LUT slice buffers | NIBUF index buffers
+    // LDS: value table(s) | position words (1 KB) | NBUF LUT slice buffers | NIBUF index buffers
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     constexpr int NBUF = sp_nbuf(GS), NIBUF = NBUF;
     constexpr int PD = NBUF - 1;  // prefetch distance of the LUT stream, in slices
+    constexpr uint32_t POS0 = sp_value_table_bytes(WIDE);  // position words
     constexpr uint32_t BUF0 = sp_table_bytes(WIDE);
     constexpr uint32_t IBUF0 = BUF0 + NBUF * SLICE;
     constexpr uint32_t IBYTES = SP_WAVES * 64 * 4 * IWORDS;   // index bytes of one slice (a 64-token block per wave)
@@ -130,9 +139,9 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel
     const uint32_t my_items = (n_items - blockIdx.x + gridDim.x - 1) / gridDim.x;
     const uint32_t total = my_items * nslices;
 
-    // Table entry c (16 bytes): value bytes of a codebook whose centroid is c (first slot of group c / 4 is 1),
-    // then the position bits (c % 4 at value slot 2 (c / 4), two bits per slot) as they stand in the low half
-    // of the lane's position word, then the same bits shifted to the high half.
+    // Table entry c (16 bytes): value bytes of a codebook whose centroid is c (first slot of group c / 4 is 1).
+    // Position table, word b: the position bits of both codebooks of index byte b (c % 4 at value slot 2 (c / 4),
+    // two bits per slot; low nibble in the low half of the word, high nibble in the high half).
     // WIDE: table h (h = 0, 1; 512 bytes each) has entry c at byte b = 16 h + c and zero entries elsewhere.
     static_assert(NW * 64 >= 256, "one table word per thread");
     if (threadIdx.x < (WIDE ? 256 : 64)) {
@@ -140,9 +149,16 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel
         const uint32_t c = b & 15, w = threadIdx.x & 3, grp = c >> 2, pos = c & 3;
         uint32_t word;
         if (w < 2) word = (grp >> 1) == w ? (1u << (16 * (grp & 1))) : 0u;  // value bytes 0..3 / 4..7: slot 2 grp
-        else word = (pos << (4 * grp)) << (w == 3 ? 16 : 0);
+        else word = 0;
         if (WIDE && (b >> 4) != table) word = 0;
         reinterpret_cast<uint32_t*>(smem)[threadIdx.x] = word;
+    }
+    if (threadIdx.x < 256) {
+        const uint32_t b = threadIdx.x;
+        auto pos_bits = [](uint32_t c) { return (c & 3u) << (4 * (c >> 2)); };
+        // WIDE: the byte is one centroid of 32; its bits belong to the half its table is looked up for
+        const uint32_t word = WIDE ? pos_bits(b & 15) << (16 * ((b >> 4) & 1)) : pos_bits(b & 15) | (pos_bits(b >> 4) << 16);
+        reinterpret_cast<uint32_t*>(smem + POS0)[b] = word;
     }
 
     auto col_of = [&](uint32_t p) { uint32_t c, t; xmap.decode(p, n_token_tiles, c, t); return c; };
@@ -234,7 +250,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel
             lds_read_u8<(i * 64 + t * 16) * 4>(raw[t][i], addr);
         });
     };
-    auto unpack_ix = [&](uint32_t (&lo)[TM][IWORDS], uint32_t (&hi)[TM][IWORDS], uint32_t (&raw)[TM][IWORDS]) {
+    auto unpack_ix = [&](uint32_t (&lo)[TM][IWORDS], uint32_t (&hi)[TM][IWORDS], uint32_t (&pa)[TM][IWORDS], uint32_t (&raw)[TM][IWORDS]) {
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
         for (int t = 0; t < TM; ++t)
@@ -251,6 +267,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel
                     lo[t][i] = (raw[t][i] << 4) & 0xF0u;
                     hi[t][i] = raw[t][i] & 0xF0u;
                 }
+                pa[t][i] = raw[t][i] << 2;  // its position word
             }
     };
 
@@ -347,9 +364,9 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel
     });
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();  // also: the table is complete
-    uint32_t iw_lo[TM][IWORDS], iw_hi[TM][IWORDS], iw_raw[TM][IWORDS];
+    uint32_t iw_lo[TM][IWORDS], iw_hi[TM][IWORDS], iw_pos[TM][IWORDS], iw_raw[TM][IWORDS];
     read_ix(iw_raw, 0);
-    unpack_ix(iw_lo, iw_hi, iw_raw);
+    unpack_ix(iw_lo, iw_hi, iw_pos, iw_raw);
 
     uint32_t item0 = blockIdx.x;
     const uint32_t b_lane = BUF0 + (g * WN + j) * 16;  // this lane's 16 bytes of codebook g, column position j
@@ -381,7 +398,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel
         // soon as its TM instructions have been issued; the sparse operand is double buffered.
         v4i b_lo[TN], b_hi[TN];
         v2i a_lo[2][TM], a_hi[2][TM];
-        v2i p_lo[2][TM], p_hi[2][TM];  // both position words of an entry: 8-byte reads of the table do not meet in a bank, 4-byte reads do
+        int pw[2][TM];  // the lane's position word
         auto issue_b = [&](auto ksc, auto cc) {
             constexpr int ks = decltype(ksc)::value, c = decltype(cc)::value;
             lds_read<((8 * ks) * WN + c * 16) * 16>(b_lo[c], bbase);
@@ -393,9 +410,8 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel
             for (int t = 0; t < TM; ++t) {
                 const uint32_t e0 = iw_lo[t][ks], e1 = iw_hi[t][ks];
                 lds_read64<0>(a_lo[ks & 1][t], e0);
-                lds_read64<8>(p_lo[ks & 1][t], e0);
                 lds_read64<0>(a_hi[ks & 1][t], e1);
-                lds_read64<8>(p_hi[ks & 1][t], e1);
+                lds_read32<POS0>(pw[ks & 1][t], iw_pos[t][ks]);
             }
         };
         // slice prologue: sparse operand first, then the dense operand of every column group, in this order
@@ -412,11 +428,11 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel
                 // ones this column group needs (see the issue order above and below)
                 if constexpr (c == 0) lgkm_wait<2 * (TN - 1)>();
                 else if constexpr (LAST) lgkm_wait<2 * (TN - 1 - c) + RI>();
-                else lgkm_wait<2 * TN + 4 * TM - 2>();
+                else lgkm_wait<2 * TN + 3 * TM - 2>();
                 if constexpr (c == 0) {
 #pragma unroll
                     for (int t = 0; t < TM; ++t)
-                        asm volatile("" : "+v"(a_lo[ks & 1][t]), "+v"(a_hi[ks & 1][t]), "+v"(p_lo[ks & 1][t]), "+v"(p_hi[ks & 1][t]));
+                        asm volatile("" : "+v"(a_lo[ks & 1][t]), "+v"(a_hi[ks & 1][t]), "+v"(pw[ks & 1][t]));
                 }
                 asm volatile("" : "+v"(b_lo[c]), "+v"(b_hi[c]));
                 __builtin_amdgcn_sched_barrier(0);
@@ -424,7 +440,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel
 #pragma unroll
                 for (int t = 0; t < TM; ++t) {
                     const v4i aa = {a_lo[ks & 1][t][0], a_lo[ks & 1][t][1], a_hi[ks & 1][t][0], a_hi[ks & 1][t][1]};
-                    acc[t][c] = __builtin_amdgcn_smfmac_i32_16x16x128_i8(aa, bb, acc[t][c], (int)(p_lo[ks & 1][t][0] | p_hi[ks & 1][t][1]), 0, 0);
+                    acc[t][c] = __builtin_amdgcn_smfmac_i32_16x16x128_i8(aa, bb, acc[t][c], pw[ks & 1][t], 0, 0);
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 if constexpr (!LAST) {
@@ -448,7 +464,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel
             lut_advance();
             if (fetch_ix) ix_advance();
         }
-        unpack_ix(iw_lo, iw_hi, iw_raw);
+        unpack_ix(iw_lo, iw_hi, iw_pos, iw_raw);
 
         copy_off = cur_off;
         cur_off = cur_off + SLICE == NBUF * SLICE ? 0 : cur_off + SLICE;
