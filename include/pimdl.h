@@ -138,7 +138,7 @@ typedef enum pimdl_gather_kernel {
     PIMDL_GATHER_AUTO = 0,
     PIMDL_GATHER_ROWS = 1,   /* byte adder: gathered row pieces summed by an identity matrix product; any C */
     PIMDL_GATHER_ONEHOT = 2, /* one-hot x table on the dense int8 matrix instruction; C <= 16 */
-    PIMDL_GATHER_SPARSE = 3  /* one-hot as a 2:4 sparse operand, 8 codebooks per instruction; 9 <= C <= 16 */
+    PIMDL_GATHER_SPARSE = 3  /* one-hot as a 2:4 sparse operand, 8 codebooks per instruction; C <= 32 (17..32 as two codebooks of 16, up to 8 as 16 with empty rows) */
 } pimdl_gather_kernel;
 typedef enum pimdl_search_kernel {
     PIMDL_SEARCH_AUTO = 0,

@@ -1271,7 +1271,7 @@ bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::s
             g->gather_kind = 1;
             break;
         case PIMDL_GATHER_SPARSE:
-            if (!(i8 && C > 8 && C <= 32)) { *why = "the sparse one-hot gather needs an int8 table with 9 to 32 centroids"; return false; }
+            if (!(i8 && C <= 32)) { *why = "the sparse one-hot gather needs an int8 table with up to 32 centroids"; return false; }
             g->gather_kind = 2;
             break;
         default: *why = "unknown gather_kernel"; return false;
@@ -1283,30 +1283,44 @@ bool plan_geometry(const pimdl_amm_desc& d, uint32_t num_cus, AmmGeom* g, std::s
         // per CU; grid_rounds) x the cost of an item of that width; among equals the widest.
         // up to 8 centroids: two codebooks share a lane's 16 K-slots (C_tile 8); 96-column tiles then do not
         // leave room for two workgroups per CU
-        const bool paired = C <= 8;
-        g->C_tile = paired ? 8 : C > 16 ? 32 : 16;
         const uint32_t slots = 2 * (num_cus ? num_cus : 256);
         const uint32_t tiles = (d.max_n + 255) / 256;
-        double best = 1e300;
+        auto pick_tn = [&](bool paired_layout) {
+            double best = 1e300;
+            uint32_t pick = 0;
+            for (uint32_t tn : {6u, 4u, 3u}) {
+                if (paired_layout && tn == 6) continue;
+                if (col_block_hint && col_block_hint != 16 * tn) continue;
+                const uint32_t blocks = (M + 16 * tn - 1) / (16 * tn);
+                const uint64_t items = (uint64_t)tiles * blocks;
+                const uint64_t items_small = (uint64_t)((d.max_n + 127) / 128) * blocks;
+                const double t256 = grid_rounds(items, slots) * item_cost(tn, false);
+                const double t128 = grid_rounds(items_small, slots) * item_cost(tn, true);
+                const double t = t128 < t256 ? t128 : t256;  // the launcher takes the better item size
+                if (t < best - 1e-9) {
+                    best = t;
+                    pick = tn;
+                }
+            }
+            return pick;
+        };
+        // Up to 8 centroids, kernel not named by the caller: the paired dense kernel has the cheaper K-loop, the
+        // sparse kernel (the table as 16 centroids with empty rows) the cheaper epilogue and the 96-column tile.
+        // Measured over N 2048..12608, K and M 768..4096, vec_len 2..8: the sparse kernel is 3 to 38 % faster where
+        // the launch is large against its codebook count (tokens x columns >= 65536 x codebooks) and either
+        // 96-column tiles are its best launch or there are at most 128 codebooks; elsewhere 0 to 20 % slower.
+        if (C <= 8 && g->gather_kind == 1 && tune.gather_kernel == PIMDL_GATHER_AUTO && !gather_dense_only() &&
+            (col_block_hint == 96 ||  // (only the sparse kernel has that tile)
+             ((uint64_t)d.max_n * M >= 65536ull * g->CB && (pick_tn(false) == 6 || g->CB <= 128))))
+            g->gather_kind = 2;
+        const bool paired = C <= 8 && g->gather_kind == 1;
+        g->C_tile = paired ? 8 : C > 16 ? 32 : 16;
         if (col_block_hint && col_block_hint != 64 && col_block_hint != 48 && (paired || col_block_hint != 96)) {
             *why = paired ? "column tile hint must be 48 or 64 for this operator"
                           : "column tile hint must be 48, 64 or 96 for this operator";
             return false;
         }
-        for (uint32_t tn : {6u, 4u, 3u}) {
-            if (paired && tn == 6) continue;
-            if (col_block_hint && col_block_hint != 16 * tn) continue;
-            const uint32_t blocks = (M + 16 * tn - 1) / (16 * tn);
-            const uint64_t items = (uint64_t)tiles * blocks;
-            const uint64_t items_small = (uint64_t)((d.max_n + 127) / 128) * blocks;
-            const double t256 = grid_rounds(items, slots) * item_cost(tn, false);
-            const double t128 = grid_rounds(items_small, slots) * item_cost(tn, true);
-            const double t = t128 < t256 ? t128 : t256;  // the launcher takes the better item size
-            if (t < best - 1e-9) {
-                best = t;
-                g->q = tn;
-            }
-        }
+        g->q = pick_tn(paired);
         g->gq = 4;
         g->cb_per_slice = 16;
         g->col_block = 16 * g->q;

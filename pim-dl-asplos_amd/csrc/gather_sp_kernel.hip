@@ -1,4 +1,5 @@
-// LUT gather-accumulate on the sparse matrix instruction (gfx950), int8 tables with 9..32 centroids.
+// LUT gather-accumulate on the sparse matrix instruction (gfx950), int8 tables with up to 32 centroids
+// (9..32 always; up to 8 where the launch rule of plan_geometry prefers it to the paired dense kernel).
 //
 // Same operator as the other gather kernels (inference-engine/src/dpu/pim_lut_kernel.c:97-2296, row-major
 // statement inference-engine/test/test_amm.cpp:164-175, epilogue inference-engine/src/host/pim_lut_host.cpp:190-203):

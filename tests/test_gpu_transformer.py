@@ -430,6 +430,27 @@ def test_every_tuning_choice_gives_the_same_bits(ctx):
             assert np.array_equal(amm.run(x).view(np.uint32), want32.view(np.uint32)), (gk, cb, st)
         assert amm.last_gather_kernel().startswith("gather_sparse" if gk == pimdl.GATHER_SPARSE else "gather_i8")
         amm.close()
+    # up to 8 centroids: the paired dense kernel (48 or 64 columns), the sparse kernel (the table as 16 centroids
+    # with empty rows; also 96 columns) or the byte adder; small launches take the paired kernel by themselves
+    for C8 in (8, 5, 1):
+        lut8 = rng.integers(-128, 128, (CB, C8, M)).astype(np.int8)
+        cent8 = rng.standard_normal((CB, C8, v)).astype(np.float32)
+        want8, _, _ = oracle.amm_cpu(x, cent8, lut8, bias, v, 0.02, 0.0, threads=8)
+        for tn in ({}, {"gather_kernel": pimdl.GATHER_ONEHOT, "col_block": 48}, {"gather_kernel": pimdl.GATHER_ONEHOT, "col_block": 64},
+                   {"gather_kernel": pimdl.GATHER_SPARSE}, {"gather_kernel": pimdl.GATHER_SPARSE, "col_block": 48},
+                   {"gather_kernel": pimdl.GATHER_SPARSE, "col_block": 64, "token_item": 128},
+                   {"gather_kernel": pimdl.GATHER_SPARSE, "col_block": 96}, {"col_block": 96},
+                   {"gather_kernel": pimdl.GATHER_SPARSE, "col_block": 48, "token_item": 512, "cb_per_slice": 64},
+                   {"gather_kernel": pimdl.GATHER_ROWS}):
+            amm = ctx.amm(cent8, lut8, np.float32(0.02), bias, max_n=N, tuning=tn)
+            assert np.array_equal(amm.run(x).view(np.uint32), want8.view(np.uint32)), (C8, tn)
+            kind = tn.get("gather_kernel", pimdl.GATHER_SPARSE if tn.get("col_block") == 96 else pimdl.GATHER_ONEHOT)
+            assert amm.last_gather_kernel().startswith({pimdl.GATHER_ONEHOT: "gather_onehot", pimdl.GATHER_SPARSE: "gather_sparse",
+                                                        pimdl.GATHER_ROWS: "gather_i8"}[kind]), (C8, tn)
+            amm.close()
+        with pytest.raises(pimdl.PimdlError) as e:
+            ctx.amm(cent8, lut8, np.float32(0.02), None, max_n=N, tuning={"gather_kernel": pimdl.GATHER_ONEHOT, "col_block": 96})
+        assert e.value.code == pimdl.ERR_INVALID
     with pytest.raises(pimdl.PimdlError):   # 33 centroids and more: the byte adder only
         ctx.amm(rng.standard_normal((CB, 40, v)).astype(np.float32), rng.integers(-128, 128, (CB, 40, M)).astype(np.int8),
                 np.float32(0.02), None, max_n=N, tuning={"gather_kernel": pimdl.GATHER_SPARSE})
