@@ -438,8 +438,8 @@ __global__ void ccs_prep_mfma_kernel(const float* __restrict__ cent, const float
     }
 }
 
-template <int V>
-__global__ __launch_bounds__(CCS_THREADS, 4) void ccs_mfma_kernel(const float* __restrict__ x,
+template <int V>  // (v = 8 does not fit four waves per SIMD: asked for two, which is what the compiler reaches)
+__global__ __launch_bounds__(CCS_THREADS, V == 8 ? 2 : 4) void ccs_mfma_kernel(const float* __restrict__ x,
                                                                  const float* __restrict__ cent,
                                                                  const float* __restrict__ aux_a,
                                                                  const float* __restrict__ cnmax_pad,
@@ -717,8 +717,11 @@ __global__ void ccs_prep_bf16_kernel(const float* __restrict__ cent, uint4* __re
     }
 }
 
+// Register budget: three waves per SIMD (168 registers) but for v = 8 with 128-token tiles and up to 16 centroids,
+// whose 64 prefetch registers do not fit: asked for three the compiler gives up and takes 288 (one workgroup per
+// CU); asked for two it takes 237 without spills, and the 76 KB of LDS allow no more than two anyway.
 template <int V, bool WIDE, int TTOK>
-__global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* __restrict__ x,
+__global__ __launch_bounds__(CCS_THREADS, (V == 8 && !WIDE && TTOK == 128) ? 2 : 3) void ccs_bf16_kernel(const float* __restrict__ x,
                                                                  const float* __restrict__ cent,
                                                                  const uint4* __restrict__ aux_b,
                                                                  const float* __restrict__ cn16,
@@ -1006,8 +1009,58 @@ __global__ __launch_bounds__(CCS_THREADS, 3) void ccs_bf16_kernel(const float* _
             }
         });
 
-        // ---- exact replay of the items that failed the margin test (rare, lane-divergent) -------
-        if (__builtin_amdgcn_ballot_w64(need != 0) != 0) {
+        // ---- exact replay of the items that failed the margin test (rare) ---------------------------------
+        // The reference's own arithmetic: per centroid the distance as a chain of single roundings, then one
+        // pass over the centroids in order that moves to a centroid closer by more than 1e-6.
+        const uint64_t replay_mask = __builtin_amdgcn_ballot_w64(need != 0);
+        constexpr int COOP_MAX = V / 2;  // up to that many lanes: one at a time, by the whole wave (8 measured the same)
+        if (replay_mask != 0 && __builtin_popcountll(WIDE ? (replay_mask & 0xFFFFFFFFull) : replay_mask) <= COOP_MAX) {
+            // A lane's replay done by the wave: lane c computes the distance to centroid c, the pass over the
+            // centroids reads them lane by lane.  A single lane doing all of it (below) keeps the other 63 waiting
+            // for C x (3v + 4) operations; this is 3v + 5C.
+            // wide: lanes l and l + 32 hold the same verdict, and lane l (h = 0) keeps the byte
+            uint64_t mask = WIDE ? (replay_mask & 0xFFFFFFFFull) : replay_mask;
+            const uint32_t wave_s = __builtin_amdgcn_readfirstlane(wave);
+            while (mask) {
+                const uint32_t l = (uint32_t)__builtin_ctzll(mask);
+                mask &= mask - 1;
+                uint32_t nd = __builtin_amdgcn_readlane(need, l);
+                const uint32_t jl = l & 31, hl = l >> 5;
+                while (nd) {
+                    const uint32_t it = (uint32_t)__builtin_ctz(nd);
+                    nd &= nd - 1;
+                    const uint32_t pl = it / TG, tg = it % TG;
+                    const uint32_t cbl = WIDE ? 2 * wave_s + pl : 2 * (2 * wave_s + pl) + hl;
+                    uint32_t bi = 0;
+                    if (tcb * RCB + cbl < CB) {
+                        const float* xo = tile + (tg * 32 + jl) * PITCH + (2 * wave_s + pl) * XSTEP + (WIDE ? 0 : V * hl);
+                        const uint32_t cl = lane < C ? lane : C - 1;  // lanes past the last centroid repeat it; never read
+                        const float* cp = cst + (cbl * C + cl) * V;
+                        float diff = __fsub_rn(xo[0], cp[0]);
+                        float d = __fmul_rn(diff, diff);
+#pragma unroll
+                        for (int t = 1; t < V; ++t) {
+                            diff = __fsub_rn(xo[t], cp[t]);
+                            d = __fadd_rn(d, __fmul_rn(diff, diff));
+                        }
+                        float best = 0.0f;
+                        for (uint32_t c = 0; c < C; ++c) {
+                            const float dc = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(d), c));
+                            const bool take = (c == 0) || (__fsub_rn(best, dc) > 1e-6f);
+                            best = take ? dc : best;
+                            bi = take ? c : bi;
+                        }
+                    }
+                    const uint32_t sh = WIDE ? 16 * (tg % 2) + 8 * pl : 16 * (tg % 2) + 8 * pl + 4 * hl;
+                    const uint32_t keep_mask = WIDE ? 255u : 15u;
+                    const bool mine = lane == l;
+#pragma unroll
+                    for (int i = 0; i < TG / 2; ++i)
+                        words[i] = (mine && tg / 2 == (uint32_t)i) ? ((words[i] & ~(keep_mask << sh)) | (bi << sh)) : words[i];
+                }
+            }
+        } else if (replay_mask != 0) {
+            // many lanes at once (ties: rows of zeros, repeated centroids): every lane replays its own items
             // kept rolled on purpose: the replay is rare and must not cost the fast path registers
 #pragma nounroll
             for (int it = 0; it < ITEMS; ++it) {
@@ -1273,7 +1326,11 @@ int launch_ccs_bf16(Ctx* ctx, const AmmGeom& g, const float* d_x, const float* d
     // compiler for four workgroups per CU with them was measured slower: 10.9 against 10.1 us at K = 768)
     // (measured 64 / 128-token tiles, us: 6.1 / 8.7 at 192 tiles; 11.0 / 11.9 at 768; 14.8 / 15.5 at 1188;
     // 17.8 / 18.8 at 1536; 28.2 .. 31.5 / 28.2 .. 29.0 at 3072; 42.3 / 41.8 at 4752)
-    const bool small_tiles = g.tune_search_tile ? g.tune_search_tile == 64 : tiles128 <= 6ull * ctx->prop.multiProcessorCount;
+    // v = 8 with up to 16 centroids: the 128-token kernel (two workgroups per CU: 237 registers, 76 KB of LDS) beats
+    // the 64-token one (three per CU, with spills) from half a tile per CU upwards (us, 64 / 128: 6.5 / 7.0 at 96
+    // tiles, 8.3 / 7.0 at 192, 15.1 / 9.7 at 512, 26 / 24.5 at 1536, 35.7 / 33.5 at 2376)
+    const uint64_t few = (V == 8 && !WIDE) ? ctx->prop.multiProcessorCount / 2 : 6ull * ctx->prop.multiProcessorCount;
+    const bool small_tiles = g.tune_search_tile ? g.tune_search_tile == 64 : tiles128 <= few;
     if (small_tiles) return launch_ccs_bf16_tt<V, WIDE, 64>(ctx, g, d_x, d_cent, d_idx, n, x_cols);
     return launch_ccs_bf16_tt<V, WIDE, 128>(ctx, g, d_x, d_cent, d_idx, n, x_cols);
 }

@@ -437,6 +437,33 @@ def test_search_with_exact_ties_and_degenerate_inputs(ctx, v, C):
     amm.close()
 
 
+@pytest.mark.parametrize("v,C", [(8, 16), (4, 16), (8, 32), (4, 32), (4, 20), (8, 12), (4, 5), (8, 8), (2, 16)])
+def test_search_with_a_few_near_ties_per_wave(ctx, v, C):
+    """One (token, codebook) pair in about 400 sits midway between two centroids, the others are ordinary: a wave
+    then has one or two lanes to replay exactly, which it does lane by lane with all its lanes (many at once take
+    another path, covered by the dense cases above).  Both token tiles of the search, a ragged batch, a codebook
+    count that leaves the last codebook tile partly empty; every index against the reference's scan."""
+    rng = np.random.default_rng(3000 + 10 * v + C)
+    N, CB = 1500, 37
+    cent = rng.standard_normal((CB, C, v)).astype(np.float32)
+    x = rng.standard_normal((N, CB, v)).astype(np.float32)
+    on = rng.random((N, CB)) < 1.0 / 400
+    a = rng.integers(0, C, (N, CB))
+    b = (a + 1 + rng.integers(0, C - 1, (N, CB))) % C
+    cbi = np.nonzero(on)[1]
+    mid = (cent[cbi, a[on]] + cent[cbi, b[on]]) * np.float32(0.5)
+    x[on] = mid + rng.standard_normal(mid.shape).astype(np.float32) * np.float32(2e-7)
+    x = x.reshape(N, CB * v)
+    want = oracle.index_calculation(x, cent, v, threads=THREADS)
+    assert (want != oracle.np_distances(x, cent).argmin(-1)).sum() > 0  # some pairs separate the scan from the true argmin
+    amm = ctx.amm(cent, np.zeros((CB, C, 4), np.int8), np.float32(1.0), None, max_n=N)
+    for tile in (0, 64, 128):
+        amm.set_tuning(search_token_tile=tile)
+        got = amm.index_calculation(x)
+        assert np.array_equal(got, want), f"tile {tile}: {(got != want).sum()} of {got.size} differ"
+    amm.close()
+
+
 @pytest.mark.parametrize("v,C", [(4, 16), (2, 16), (8, 16), (4, 32)])
 def test_search_with_non_finite_values(ctx, v, C):
     """NaN / Inf / near-overflow values in activations and centroids take the exact path and match
