@@ -30,8 +30,8 @@ MFMA_I8_PEAK_TOPS = 5000.0                 # MI355X dense int8 matrix peak
 # FETCH_SIZE is scaled by 2.0 and WRITE_SIZE by 1.0: what a streaming copy of known size reads for the same
 # counters in the same runs.
 MEASURED_GATHER_TRAFFIC = {
-    ("gather_sparse_kernel<6, 4, 16, 4, false>", 8192, 768, 3072): {"fetch_kib": 9809.1, "write_kib": 98306.3},
-    ("gather_sparse_kernel<3, 4, 64, 8, false>", 8192, 3072, 768): {"fetch_kib": 15644.5, "write_kib": 25007.5},
+    ("gather_sparse_kernel<6, 4, 16, 4, false>", 8192, 768, 3072): {"fetch_kib": 9815.5, "write_kib": 98309.6},
+    ("gather_sparse_kernel<3, 4, 64, 8, false>", 8192, 3072, 768): {"fetch_kib": 15644.5, "write_kib": 25039.7},
 }
 FETCH_SCALE, WRITE_SCALE = 2.0, 1.0
 CLOCK_SETTLE_S = 0.08                      # untimed pre-heat: the engine clock needs ~20 ms of this load to ramp up
