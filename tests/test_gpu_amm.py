@@ -284,6 +284,8 @@ def test_two_tokens_per_lane_in_the_fp32_table_gather(ctx, kind):
     (257, 256, 2, 32, (100, 60), "i8"),         # 32 centroids: byte indices, tiled index rows (sparse gather, two tables)
     (900, 256, 4, 32, (96, 96, 96), "i8"),      # 32 centroids, three members in one gather launch
     (300, 256, 8, 16, (48, 80, 48), "f32"),     # fp32 tables
+    (8192, 768, 4, 8, (768, 3072), "i8"),       # 8 centroids at a size where the wide member takes the sparse kernel, the narrow one the paired
+    (8192, 256, 8, 8, (1536, 1536), "i8"),      # 8 centroids, both members on the sparse kernel, one gather launch
 ])
 def test_operators_sharing_an_input_are_searched_by_one_launch(ctx, N, K, v, C, Ms, lut):
     """AmmGroup (separate Q/K/V projections): every output bit for bit that of the operator run alone."""
@@ -299,6 +301,10 @@ def test_operators_sharing_an_input_are_searched_by_one_launch(ctx, N, K, v, C, 
     outs = group.run(x)
     for a, o in zip(amms, outs):
         assert np.array_equal(o.view(np.uint32), a.run(x).view(np.uint32))
+    if C == 8 and N == 8192:  # which kernel each member's launch rule took
+        want_kernels = {(768, 3072): ("gather_onehot", "gather_sparse"), (1536, 1536): ("gather_sparse", "gather_sparse")}[Ms]
+        for a, k in zip(amms, want_kernels):
+            assert a.last_gather_kernel().startswith(k), (a.last_gather_kernel(), k)
     outs2 = group.run(x[:77])  # a smaller batch through the same group
     for o, o2 in zip(outs, outs2):
         assert np.array_equal(o[:77], o2)
