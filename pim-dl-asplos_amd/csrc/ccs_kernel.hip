@@ -979,7 +979,7 @@ __global__ __launch_bounds__(CCS_THREADS, (V == 8 && !WIDE && TTOK == 128) ? 2 :
             uint32_t bi = __float_as_uint(m1) & 15u;
             if constexpr (WIDE) {
                 // the other 16 centroids of the codebook were searched by lane l ^ 32: both lanes merge the
-                // two (smallest, second smallest) pairs and reach the same verdict.  Equal tagged minima
+                // two (smallest, second smallest) pairs and reach the same outcome.  Equal tagged minima
                 // give m2 == m1, which fails the margin test.
                 const auto s1 = __builtin_amdgcn_permlane32_swap(__float_as_uint(m1), __float_as_uint(m1), false, false);
                 const auto s2 = __builtin_amdgcn_permlane32_swap(__float_as_uint(m2), __float_as_uint(m2), false, false);
@@ -1018,7 +1018,7 @@ __global__ __launch_bounds__(CCS_THREADS, (V == 8 && !WIDE && TTOK == 128) ? 2 :
             // A lane's replay done by the wave: lane c computes the distance to centroid c, the pass over the
             // centroids reads them lane by lane.  A single lane doing all of it (below) keeps the other 63 waiting
             // for C x (3v + 4) operations; this is 3v + 5C.
-            // wide: lanes l and l + 32 hold the same verdict, and lane l (h = 0) keeps the byte
+            // wide: lanes l and l + 32 hold the same outcome, and lane l (h = 0) keeps the byte
             uint64_t mask = WIDE ? (replay_mask & 0xFFFFFFFFull) : replay_mask;
             const uint32_t wave_s = __builtin_amdgcn_readfirstlane(wave);
             while (mask) {
