@@ -8,6 +8,15 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 
+# Switches of the environment that keep one kernel for every shape (for comparing kernels: same results, other
+# launches).  Assertions about WHICH kernel a shape takes hold for the library's own choice only.
+KERNEL_SWITCHES = ("PIMDL_CCS_EXACT", "PIMDL_CCS_F32", "PIMDL_GATHER_ROWS", "PIMDL_GATHER_DENSE")
+
+
+def kernel_switches():
+    return [e for e in KERNEL_SWITCHES if os.environ.get(e) == "1"]
+
+
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 

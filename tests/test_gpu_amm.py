@@ -9,6 +9,7 @@ import numpy as np
 import pytest
 
 import oracle
+from conftest import kernel_switches
 from __graft_entry__ import load_package
 
 pimdl = load_package()
@@ -289,7 +290,7 @@ def test_two_tokens_per_lane_in_the_fp32_table_gather(ctx, kind):
 ])
 def test_operators_sharing_an_input_are_searched_by_one_launch(ctx, N, K, v, C, Ms, lut):
     """AmmGroup (separate Q/K/V projections): every output bit for bit that of the operator run alone."""
-    if any(os.environ.get(e) == "1" for e in ("PIMDL_CCS_EXACT", "PIMDL_CCS_F32", "PIMDL_GATHER_ROWS")):
+    if kernel_switches():
         pytest.skip("a kernel this test is about is switched off by the environment")
     rng = np.random.default_rng(N + K)
     x = rng.standard_normal((N, K)).astype(np.float32)
@@ -323,7 +324,7 @@ def test_operators_sharing_an_input_are_searched_by_one_launch(ctx, N, K, v, C, 
 
 
 def test_group_conditions(ctx):
-    if any(os.environ.get(e) == "1" for e in ("PIMDL_CCS_EXACT", "PIMDL_CCS_F32", "PIMDL_GATHER_ROWS")):
+    if kernel_switches():
         pytest.skip("a kernel this test is about is switched off by the environment")
     rng = np.random.default_rng(5)
     mk = lambda K, v, C, M, kind="i8": ctx.amm(*(lambda c: (c[1], c[2]))(make_case(1, 1, K, v, C, M, kind)),
