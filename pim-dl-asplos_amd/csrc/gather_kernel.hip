@@ -116,7 +116,7 @@ __device__ __forceinline__ void load_idx_async(uint32_t& reg, const void* gptr)
 // path nor the LDS write port ever sees a burst, no wave ever stalls on issue, and the only
 // synchronisation is one barrier per slice between waves that all did identical work.
 template <int C_T, int Q, int GQ, int TG, int IDX_BITS>
-__global__ __launch_bounds__(GATHER_THREADS, 4) void gather_i8_kernel(
+__global__ __launch_bounds__(GATHER_THREADS, TG == 4 ? 2 : 4) void gather_i8_kernel(
     const uint8_t* __restrict__ idx, const int8_t* __restrict__ lut, float* __restrict__ out,
     int32_t* __restrict__ acc_out, uint32_t N, uint32_t M, uint32_t CB_pad, uint32_t idx_row_bytes,
     uint32_t n_token_tiles, uint32_t n_items, Epilogue ep)
@@ -294,8 +294,13 @@ __global__ __launch_bounds__(GATHER_THREADS, 4) void gather_i8_kernel(
         // slice k+1, the indices fetched during the previous iteration have landed
         // (the indices move out of their in-flight registers inside the asm, behind the wait, so the
         // compiler never holds a value it could copy before it has landed)
-        static_assert(TG == 1 || TG == 2, "operand list of the wait below");
-        if constexpr (TG == 2)
+        static_assert(TG == 1 || TG == 2 || TG == 4, "operand list of the wait below");
+        if constexpr (TG == 4)
+            asm volatile("s_waitcnt vmcnt(0)\n\tv_mov_b32 %0, %4\n\tv_mov_b32 %1, %5\n\tv_mov_b32 %2, %6\n\tv_mov_b32 %3, %7"
+                         : "=&v"(idx_cur[0]), "=&v"(idx_cur[1]), "=&v"(idx_cur[2]), "=&v"(idx_cur[3])
+                         : "v"(idx_nxt[0]), "v"(idx_nxt[1]), "v"(idx_nxt[2]), "v"(idx_nxt[3])
+                         : "memory");
+        else if constexpr (TG == 2)
             asm volatile("s_waitcnt vmcnt(0)\n\tv_mov_b32 %0, %2\n\tv_mov_b32 %1, %3"
                          : "=&v"(idx_cur[0]), "=&v"(idx_cur[1])
                          : "v"(idx_nxt[0]), "v"(idx_nxt[1])
@@ -1410,6 +1415,13 @@ int launch_gather(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, in
             }
             return set_error(ctx, PIMDL_ERR_UNSUPPORTED, "no one-hot gather kernel for %u column groups", g.q);
         }
+        // 64 centroids and more: a slice holds few codebooks (8, 8, 4), so an item's time goes to its slices'
+        // barriers and staging as much as to its reads; four token groups per wave (256-token items) halve the
+        // slices per token where the batch still gives every resident workgroup two items (measured at N = 8192,
+        // 768 -> 3072: C = 64 145 -> 140 us, C = 128 237 -> 186, C = 256 416 -> 338; with fewer items, 3072 -> 768
+        // at C = 256, 407 -> 434)
+        const uint64_t items4 = (uint64_t)((n + 255) / 256) * (g.M_pad / g.col_block);
+        const bool tg4 = g.C_tile >= 64 && items4 >= 4ull * ctx->prop.multiProcessorCount;
         switch (g.C_tile) {
             case 8: return launch_i8<8, 4, 8, 2, 4>(ctx, a, d_idx, d_out, d_acc, n, ep);
             case 16:
@@ -1419,10 +1431,17 @@ int launch_gather(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, in
                 return g.q == 3 ? launch_i8<32, 3, 4, 2, 8>(ctx, a, d_idx, d_out, d_acc, n, ep)
                                 : launch_i8<32, 4, 4, 2, 8>(ctx, a, d_idx, d_out, d_acc, n, ep);
             case 64:
+                if (tg4)
+                    return g.q == 3 ? launch_i8<64, 3, 2, 4, 8>(ctx, a, d_idx, d_out, d_acc, n, ep)
+                                    : launch_i8<64, 4, 2, 4, 8>(ctx, a, d_idx, d_out, d_acc, n, ep);
                 return g.q == 3 ? launch_i8<64, 3, 2, 2, 8>(ctx, a, d_idx, d_out, d_acc, n, ep)
                                 : launch_i8<64, 4, 2, 2, 8>(ctx, a, d_idx, d_out, d_acc, n, ep);
-            case 128: return launch_i8<128, 2, 2, 2, 8>(ctx, a, d_idx, d_out, d_acc, n, ep);
-            case 256: return launch_i8<256, 2, 1, 2, 8>(ctx, a, d_idx, d_out, d_acc, n, ep);
+            case 128:
+                return tg4 ? launch_i8<128, 2, 2, 4, 8>(ctx, a, d_idx, d_out, d_acc, n, ep)
+                           : launch_i8<128, 2, 2, 2, 8>(ctx, a, d_idx, d_out, d_acc, n, ep);
+            case 256:
+                return tg4 ? launch_i8<256, 2, 1, 4, 8>(ctx, a, d_idx, d_out, d_acc, n, ep)
+                           : launch_i8<256, 2, 1, 2, 8>(ctx, a, d_idx, d_out, d_acc, n, ep);
         }
     } else {
         switch (g.C_tile) {

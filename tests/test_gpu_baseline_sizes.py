@@ -93,8 +93,9 @@ ENVELOPE = (
     [(f"bert-base-v{v}-qkv", 2048, 768, v, 16, 2304) for v in (2, 4, 8, 16, 32)] +
     [(f"bert-base-ct{c}-ffn2", 2048, 3072, 4, c, 768) for c in (8, 16, 32, 64, 128)] +
     # centroid counts between the configurations' powers of two (17..32 run as two codebooks of 16 side by side;
-    # 5 and 8 at this width run on the sparse kernel as 16 with empty rows)
-    [(f"bert-base-ct{c}-ffn1", 8192, 768, 4, c, 3072) for c in (5, 8, 12, 20, 24)] +
+    # 5 and 8 at this width run on the sparse kernel as 16 with empty rows; 64 and more on the byte adder with
+    # 256-token items at this size)
+    [(f"bert-base-ct{c}-ffn1", 8192, 768, 4, c, 3072) for c in (5, 8, 12, 20, 24, 64, 128, 200)] +
     [("vit-huge-ffn1", 2112, 1280, 4, 16, 5120), ("vit-huge-ffn2", 2112, 5120, 4, 16, 1280)])
 
 
