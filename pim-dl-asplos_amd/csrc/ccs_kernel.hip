@@ -242,6 +242,10 @@ __global__ __launch_bounds__(CCS_THREADS) void ccs_kernel(const float* __restric
     constexpr bool PREFETCH = FAST && IDX_BITS == 4;  // C <= 16: one group per codebook
     float am_ring[2][V + 1];
     if constexpr (PREFETCH) load_aux(am_ring[0], cb0, 0);
+    // more than 16 centroids: the operands of the next group of 16 (of this codebook or the next) are requested
+    // before the current group is scanned, so a group's scan covers the next one's loads
+    float am_cur[V + 1], am_nxt[V + 1];
+    if constexpr (FAST && !PREFETCH) load_aux(am_cur, cb0, 0);
 
     static_for<CBT>([&](auto cbl_c) {
         constexpr int cbl = decltype(cbl_c)::value;
@@ -276,9 +280,11 @@ __global__ __launch_bounds__(CCS_THREADS) void ccs_kernel(const float* __restric
                 scan16(am_ring[cbl & 1], 0);
             } else {
                 for (uint32_t grp = 0; grp < groups; ++grp) {
-                    float am[V + 1];
-                    load_aux(am, cb, grp);
-                    scan16(am, 16 * grp);
+                    const bool last = grp + 1 == groups;
+                    load_aux(am_nxt, last ? cb + 1 : cb, last ? 0 : grp + 1);
+                    scan16(am_cur, 16 * grp);
+#pragma unroll
+                    for (int t = 0; t <= V; ++t) am_cur[t] = am_nxt[t];
                 }
             }
             bi = __float_as_uint(m1) & ID_MASK;
