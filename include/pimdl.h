@@ -186,7 +186,12 @@ PIMDL_API int pimdl_amm_destroy(pimdl_amm* amm);
  *   in   fp32 [n][K], host or device
  *   out  fp32 [n][M], host or device
  * Synchronous for host pointers.  For device pointers the kernels are queued on the context's
- * stream and the call returns at once; use pimdl_synchronize() or stream ordering. */
+ * stream and the call returns at once; use pimdl_synchronize() or stream ordering.
+ * Host buffers may be ordinary pageable memory: the batch is cut into chunks of tokens that are copied into
+ * pinned staging buffers by a pool of host threads (PIMDL_COPY_THREADS, default 8), transferred, searched,
+ * gathered, transferred back and copied out with four chunks in flight, so the copies overlap each other and
+ * the kernels; the output bits are those of one launch over the whole batch.  With `out` on the device and
+ * `in` on the host the call returns once `in` has been copied (it may be reused); the rest is stream-ordered. */
 PIMDL_API int pimdl_amm_run(pimdl_amm* amm, const float* in, uint32_t n, float* out);
 
 /* pimdl_amm_run for callers that cannot allocate device memory (code under HIP graph capture, tight serving
@@ -276,6 +281,19 @@ typedef struct pimdl_tiling {
 /* amm_host with the reference's output order.  in host or device; out host or device. */
 PIMDL_API int pimdl_amm_run_tiled(pimdl_amm* amm, const float* in, uint32_t n, float* out,
                                   const pimdl_tiling* tiling);
+/* pimdl_amm_run_tiled with the phases run one after the other and waited for, and their wall-clock seconds
+ * ADDED to *acc: the counterpart of the reference's AMM_BREAKDOWN build, which accumulates
+ * "index calculation time" (src/host/amm_host.cpp:14-26) and "other / data transfer / pim kernel latency"
+ * (src/host/pim_lut_host.cpp:124-212) the same way, with a dpu_sync between phases.  Slower than
+ * pimdl_amm_run_tiled (nothing overlaps); same output bits. */
+typedef struct pimdl_amm_breakdown {
+    double h2d_s;    /* input to the device (staging included) */
+    double search_s; /* closest-centroid search kernel: the reference's index calculation */
+    double gather_s; /* LUT gather-accumulate kernel (+ output re-tiling): the reference's pim kernel */
+    double d2h_s;    /* output back to the host */
+} pimdl_amm_breakdown;
+PIMDL_API int pimdl_amm_run_breakdown(pimdl_amm* amm, const float* in, uint32_t n, float* out,
+                                      const pimdl_tiling* tiling, pimdl_amm_breakdown* acc);
 /* pim_lut with the reference's index and output orders.  idx is HOST uint16 centroid ids. */
 PIMDL_API int pimdl_lut_gather_tiled(pimdl_amm* amm, const uint16_t* idx, uint32_t n, float* out,
                                      const pimdl_tiling* tiling);

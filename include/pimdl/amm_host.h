@@ -21,8 +21,10 @@
 // Differences from the reference, all deliberate:
 //   * the LUT and the centroids are uploaded to the device once per (pointer, shape) and reused; the
 //     reference re-sends the LUT on every call (pim_lut_host.cpp:143).  Every call hashes both buffers
-//     in full (one pass over host memory) and uploads again when anything behind the pointers has
-//     changed; bias_tensor is sent on every call, as the reference reads it on every call (:201).
+//     in full (one pass over host memory, on the library's host threads) and uploads again when anything
+//     behind the pointers has changed (PimdlHostOptions::assume_unchanged skips the hash); bias_tensor is
+//     compared with the device's copy on every call and sent when it differs (the reference reads it on
+//     every call, :201).
 //     pimdl_host_invalidate(lut_table) drops the device copy explicitly.
 //   * failures throw std::runtime_error (the reference aborts through DPU_ASSERT);
 //   * nothing is leaked per call (the reference leaks its index and int32 buffers,
@@ -59,7 +61,21 @@ void amm_host(dpu_set_t* dpu_set, float* input_tensor, float* centroid_tensor, l
 struct PimdlHostOptions {
     bool mutate_index_buffer = true;  // pim_lut(): reproduce the reference's in-place index rewrite
     int device = 0;                   // GPU used by allocate_dpu / by index_calculation's implicit context
+    // amm_host / pim_lut: trust the device copy of a LUT and its centroids once they have been uploaded for a
+    // (pointer, shape) and skip the per-call hash of both buffers.  Off by default: the reference re-sends the LUT
+    // on every call (pim_lut_host.cpp:143), so in-place edits must be seen.  With it on, edits behind the same
+    // pointers go unnoticed until pimdl_host_invalidate(lut_table).
+    bool assume_unchanged = false;
+    // amm_host: run the phases one after the other, add their wall-clock seconds to pimdl_host_profiles() and
+    // print the two lines of the reference's AMM_BREAKDOWN build (amm_host.cpp:14-26, pim_lut_host.cpp:211).
+    bool breakdown = false;
 };
 PimdlHostOptions& pimdl_host_options();
+// The reference's amm_profiles (utils.h:37-40), seconds, cumulative: index calculation = the search kernel,
+// kernel = the gather kernel, data transfer = input to and output from the device, other = the rest of the call.
+struct PimdlHostProfiles {
+    double index_calc_latency = 0, other_latency = 0, data_transfer_latency = 0, kernel_latency = 0;
+};
+PimdlHostProfiles& pimdl_host_profiles();
 // Forget the device copy of a LUT (and its centroids) cached under this host pointer.
 void pimdl_host_invalidate(const void* lut_table);

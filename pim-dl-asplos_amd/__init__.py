@@ -33,7 +33,7 @@ EXPORTS = ["pimdl_init", "pimdl_destroy", "pimdl_last_error", "pimdl_set_stream"
            "pimdl_diag_mfma_error", "pimdl_amm_group_create", "pimdl_amm_group_run", "pimdl_amm_group_destroy",
            "pimdl_attention", "pimdl_amm_group_fused_cols", "pimdl_amm_group_run_fused", "pimdl_amm_run_noalloc", "pimdl_amm_set_bias",
            "pimdl_amm_create_with", "pimdl_amm_set_tuning", "pimdl_amm_get_tuning", "pimdl_lutgen_mode",
-           "pimdl_diag_mfma_error_crafted", "pimdl_amm_last_gather_kernel"]
+           "pimdl_diag_mfma_error_crafted", "pimdl_amm_last_gather_kernel", "pimdl_amm_run_breakdown"]
 NOALLOC_SCRATCH_BYTES = 8 << 20
 
 

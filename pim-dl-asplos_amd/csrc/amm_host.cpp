@@ -2,14 +2,17 @@
 // Plain host code: everything that touches the GPU goes through include/pimdl.h.
 #include "pimdl/amm_host.h"
 
+#include <stdio.h>
 #include <string.h>
 
+#include <chrono>
 #include <map>
 #include <mutex>
 #include <stdexcept>
 #include <tuple>
 #include <vector>
 
+#include "host_pool.h"
 #include "pimdl.h"
 
 #define PIMDL_HOST_API __attribute__((visibility("default")))
@@ -30,6 +33,9 @@ std::mutex g_mu;
 std::map<std::pair<pimdl_ctx*, Key>, Cached> g_cache;
 pimdl_ctx* g_implicit_ctx = nullptr;
 PimdlHostOptions g_opts;
+PimdlHostProfiles g_profiles;
+
+double now_s() { return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count(); }
 
 [[noreturn]] void fail(pimdl_ctx* ctx, const char* what)
 {
@@ -51,7 +57,26 @@ pimdl_ctx* implicit_ctx()
 // Hash of every byte (four independent multiply-xor lanes over 32-byte blocks, then the tail): one pass over
 // memory, a fraction of the host-to-device copy that it saves.  The reference re-sends LUT and centroids on
 // every call, so whatever the caller changed behind the same pointers must be noticed here.
+uint64_t fingerprint_piece(const void* p, size_t bytes);
+
+// The pieces of a large buffer are hashed side by side on the host thread pool and their hashes combined in order.
 uint64_t fingerprint(const void* p, size_t bytes)
+{
+    constexpr size_t PIECE = 1u << 20;
+    if (bytes <= PIECE) return fingerprint_piece(p, bytes);
+    const size_t pieces = (bytes + PIECE - 1) / PIECE;
+    std::vector<uint64_t> h(pieces);
+    const int width = pimdl::host_pool().width();
+    pimdl::host_pool().run(width, [&](int w) {
+        for (size_t i = w; i < pieces; i += width) {
+            const size_t off = i * PIECE, len = off + PIECE <= bytes ? PIECE : bytes - off;
+            h[i] = fingerprint_piece(static_cast<const unsigned char*>(p) + off, len);
+        }
+    });
+    return fingerprint_piece(h.data(), pieces * sizeof(uint64_t)) ^ bytes;
+}
+
+uint64_t fingerprint_piece(const void* p, size_t bytes)
 {
     const unsigned char* b = static_cast<const unsigned char*>(p);
     const uint64_t m = 0x9E3779B97F4A7C15ull;
@@ -101,15 +126,23 @@ pimdl_amm* get_operator(pimdl_ctx* ctx, const float* centroids, uint32_t K, uint
     memcpy(&bias_bits, &lp.bias, 4);
     const Key key(lut, centroids, K, v, C, M, ft, scale_bits, bias_bits);
     const size_t lut_bytes = (size_t)CB * C * M;
-    const uint64_t fp = fingerprint(lut, lut_bytes) ^ (centroids ? fingerprint(centroids, (size_t)CB * C * v * 4) : 0);
 
     std::lock_guard<std::mutex> lock(g_mu);
     auto it = g_cache.find(std::make_pair(ctx, key));
+    // assume_unchanged: a cached operator is trusted without reading the caller's tables again
+    const bool trust = g_opts.assume_unchanged && it != g_cache.end();
+    const uint64_t fp = trust ? it->second.fingerprint
+                              : fingerprint(lut, lut_bytes) ^ (centroids ? fingerprint(centroids, (size_t)CB * C * v * 4) : 0);
+    uint32_t max_n = lp.n;
     if (it != g_cache.end()) {
         if (it->second.fingerprint == fp && it->second.max_n >= lp.n) {
-            if (pimdl_amm_set_bias(it->second.amm, bias)) fail(ctx, "pimdl_amm_set_bias");
+            if (pimdl_amm_set_bias(it->second.amm, bias)) fail(ctx, "pimdl_amm_set_bias");  // a no-op unless it changed
             return it->second.amm;
         }
+        // a batch that creeps upwards: room for half as much again, so that operators are rebuilt (and the
+        // table sent again) a logarithmic number of times
+        if (it->second.fingerprint == fp && it->second.max_n < lp.n && it->second.max_n + it->second.max_n / 2 > lp.n)
+            max_n = it->second.max_n + it->second.max_n / 2;
         pimdl_amm_destroy(it->second.amm);
         g_cache.erase(it);
     }
@@ -127,7 +160,7 @@ pimdl_amm* get_operator(pimdl_ctx* ctx, const float* centroids, uint32_t K, uint
     }
     pimdl_amm_desc d;
     memset(&d, 0, sizeof(d));
-    d.max_n = lp.n;
+    d.max_n = max_n;
     d.input_feature_len = K;
     d.sub_vec_len = v;
     d.num_centroid = C;
@@ -138,7 +171,7 @@ pimdl_amm* get_operator(pimdl_ctx* ctx, const float* centroids, uint32_t K, uint
     d.lut_bias = lp.bias;
     pimdl_amm* amm = nullptr;
     if (pimdl_amm_create(ctx, &d, centroids, canon_ptr, &lp.scale, bias, &amm)) fail(ctx, "pimdl_amm_create");
-    g_cache[std::make_pair(ctx, key)] = Cached{amm, fp, lp.n};
+    g_cache[std::make_pair(ctx, key)] = Cached{amm, fp, max_n};
     return amm;
 }
 
@@ -175,6 +208,7 @@ void mutate_index(const LUTParams& lp, index_data_type* idx)
 }  // namespace
 
 PIMDL_HOST_API PimdlHostOptions& pimdl_host_options() { return g_opts; }
+PIMDL_HOST_API PimdlHostProfiles& pimdl_host_profiles() { return g_profiles; }
 
 PIMDL_HOST_API void pimdl_host_invalidate(const void* lut_table)
 {
@@ -251,7 +285,23 @@ PIMDL_HOST_API void amm_host(dpu_set_t* dpu_set, float* input_tensor, float* cen
     if (ip.n != lp.n || ip.num_codebook != lp.num_codebook || ip.num_centroid != lp.num_centroid ||
         ip.input_feature_len != ip.num_codebook * ip.sub_vec_len)
         throw std::runtime_error("amm_host: index_params and lut_params disagree");
+    const double t0 = g_opts.breakdown ? now_s() : 0.0;
     pimdl_amm* amm = get_operator(ctx, centroid_tensor, ip.input_feature_len, ip.sub_vec_len, lut_table, bias_tensor, lp);
     const pimdl_tiling t = tiling_of(lp);
-    if (pimdl_amm_run_tiled(amm, input_tensor, lp.n, output_tensor, &t)) fail(ctx, "amm_host");
+    if (!g_opts.breakdown) {
+        if (pimdl_amm_run_tiled(amm, input_tensor, lp.n, output_tensor, &t)) fail(ctx, "amm_host");
+        return;
+    }
+    // The reference's AMM_BREAKDOWN build (amm_host.cpp:14-26, pim_lut_host.cpp:124-212): cumulative buckets,
+    // printed on every call in the reference's own words.
+    pimdl_amm_breakdown b = {0, 0, 0, 0};
+    if (pimdl_amm_run_breakdown(amm, input_tensor, lp.n, output_tensor, &t, &b)) fail(ctx, "amm_host");
+    const double total = now_s() - t0;
+    g_profiles.index_calc_latency += b.search_s;
+    g_profiles.data_transfer_latency += b.h2d_s + b.d2h_s;
+    g_profiles.kernel_latency += b.gather_s;
+    g_profiles.other_latency += total - (b.search_s + b.h2d_s + b.d2h_s + b.gather_s);
+    printf("index calculation time %.6f\n", g_profiles.index_calc_latency);
+    printf("other latency %.6f, data transfer latency %.6f, pim kernel latency %.6f\n", g_profiles.other_latency,
+           g_profiles.data_transfer_latency, g_profiles.kernel_latency);
 }

@@ -815,14 +815,7 @@ int launch_onehot_tm(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out,
     static_assert(2 * LDS <= 160 * 1024, "two workgroups per CU");
     constexpr int OH_TOK_ITEM = oh_tok_item(TM);
     auto kern = gather_onehot_kernel<TN, TM, P8, GS>;
-    static bool attr_set = false;
-    if (!attr_set) {
-        int rc = hip_check(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                                    hipFuncAttributeMaxDynamicSharedMemorySize, LDS),
-                           "hipFuncSetAttribute(gather_onehot)");
-        if (rc) return rc;
-        attr_set = true;
-    }
+    if (int rc = allow_dynamic_lds(ctx, reinterpret_cast<const void*>(kern), LDS, "hipFuncSetAttribute(gather_onehot)")) return rc;
     const uint32_t n_token_tiles = (n + OH_TOK_ITEM - 1) / OH_TOK_ITEM;
     const uint32_t n_items = n_token_tiles * (a.g.M_pad / (16 * TN));
     uint32_t grid = ctx->prop.multiProcessorCount * 2;  // two workgroups per CU, see plan_geometry
@@ -1069,14 +1062,7 @@ int launch_i8(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_
     constexpr int PITCH = 16 * (Q | 1);
     constexpr int LDS = 2 * 4 * GQ * C_T * PITCH;
     auto kern = gather_i8_kernel<C_T, Q, GQ, TG, IDX_BITS>;
-    static bool attr_set = false;
-    if (!attr_set) {
-        int rc = hip_check(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                                    hipFuncAttributeMaxDynamicSharedMemorySize, LDS),
-                           "hipFuncSetAttribute(gather_i8)");
-        if (rc) return rc;
-        attr_set = true;
-    }
+    if (int rc = allow_dynamic_lds(ctx, reinterpret_cast<const void*>(kern), LDS, "hipFuncSetAttribute(gather_i8)")) return rc;
     const uint32_t n_token_tiles = (n + TOK_ITEM - 1) / TOK_ITEM;
     const uint32_t n_items = n_token_tiles * (a.g.M_pad / (16 * Q));
     // persistent grid: as many workgroups as fit at once (LDS-limited), never more than there are items
@@ -1096,14 +1082,7 @@ int launch_f32_impl(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, 
 {
     constexpr int LDS = 2 * GS * C_T * (f32_lut_chunked(C_T, Q) ? 16 * Q : 16 * Q + 16);
     auto kern = gather_f32_kernel<C_T, Q, GS, IDX_BITS, GROUPED, TPL>;
-    static bool attr_set = false;
-    if (!attr_set) {
-        int rc = hip_check(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                                    hipFuncAttributeMaxDynamicSharedMemorySize, LDS),
-                           "hipFuncSetAttribute(gather_f32)");
-        if (rc) return rc;
-        attr_set = true;
-    }
+    if (int rc = allow_dynamic_lds(ctx, reinterpret_cast<const void*>(kern), LDS, "hipFuncSetAttribute(gather_f32)")) return rc;
     const uint32_t n_token_tiles = (n + GF_THREADS * TPL - 1) / (GF_THREADS * TPL), colblocks = a.g.M_pad / (4 * Q);
     const uint64_t wgs = (uint64_t)n_token_tiles * colblocks;
     if (wgs > 0x7FFFFFFFull) return set_error(ctx, PIMDL_ERR_UNSUPPORTED, "gather: %llu workgroups", (unsigned long long)wgs);
@@ -1416,12 +1395,13 @@ int launch_gather(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, in
             return set_error(ctx, PIMDL_ERR_UNSUPPORTED, "no one-hot gather kernel for %u column groups", g.q);
         }
         // 64 centroids and more: a slice holds few codebooks (8, 8, 4), so an item's time goes to its slices'
-        // barriers and staging as much as to its reads; four token groups per wave (256-token items) halve the
-        // slices per token where the batch still gives every resident workgroup two items (measured at N = 8192,
-        // 768 -> 3072: C = 64 145 -> 140 us, C = 128 237 -> 186, C = 256 416 -> 338; with fewer items, 3072 -> 768
-        // at C = 256, 407 -> 434)
-        const uint64_t items4 = (uint64_t)((n + 255) / 256) * (g.M_pad / g.col_block);
-        const bool tg4 = g.C_tile >= 64 && items4 >= 4ull * ctx->prop.multiProcessorCount;
+        // barriers and staging as much as to its reads; four token groups per wave (items of 8 waves x 64 = 512
+        // tokens instead of 256) halve the slices per token where the batch still gives every resident workgroup
+        // (two per CU) such an item (measured at N = 8192, 768 -> 3072: C = 64 145 -> 140 us, C = 128 237 -> 186,
+        // C = 256 416 -> 338; with fewer items, 3072 -> 768 at C = 256, 407 -> 434)
+        constexpr uint32_t TOK_ITEM4 = GATHER_WAVES * 4 * 16;
+        const uint64_t items4 = (uint64_t)((n + TOK_ITEM4 - 1) / TOK_ITEM4) * (g.M_pad / g.col_block);
+        const bool tg4 = g.C_tile >= 64 && items4 >= 2ull * ctx->prop.multiProcessorCount;
         switch (g.C_tile) {
             case 8: return launch_i8<8, 4, 8, 2, 4>(ctx, a, d_idx, d_out, d_acc, n, ep);
             case 16:

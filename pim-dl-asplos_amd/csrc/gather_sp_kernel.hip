@@ -485,14 +485,7 @@ int launch_sparse_tm(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out,
     constexpr int TOK_ITEM = sp_tok_item(TM, NW);
     auto kern = gather_sparse_kernel<TN, TM, GS, NW, WIDE>;
     const uint32_t cb16 = sparse_codebooks(a.g);  // codebooks of 16 centroids in the tiled table
-    static bool attr_set = false;
-    if (!attr_set) {
-        int rc = hip_check(ctx, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                                    hipFuncAttributeMaxDynamicSharedMemorySize, LDS),
-                           "hipFuncSetAttribute(gather_sparse)");
-        if (rc) return rc;
-        attr_set = true;
-    }
+    if (int rc = allow_dynamic_lds(ctx, reinterpret_cast<const void*>(kern), LDS, "hipFuncSetAttribute(gather_sparse)")) return rc;
     const uint32_t n_token_tiles = (n + TOK_ITEM - 1) / TOK_ITEM;
     const uint32_t n_items = n_token_tiles * (a.g.M_pad / (16 * TN));
     uint32_t grid = ctx->prop.multiProcessorCount * (NW == 4 ? 2 : 1);

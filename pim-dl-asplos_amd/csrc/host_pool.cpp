@@ -1,0 +1,137 @@
+// The process-wide host thread pool (host_pool.h).  Plain host code.
+#include "host_pool.h"
+
+#include <stdlib.h>
+#include <string.h>
+
+#include <condition_variable>
+#include <mutex>
+#include <thread>
+#include <vector>
+
+namespace pimdl {
+namespace {
+
+class Pool final : public HostPool {
+public:
+    explicit Pool(int width) : width_(width < 1 ? 1 : width)
+    {
+        for (int i = 1; i < width_; ++i) workers_.emplace_back([this] { loop(); });
+    }
+    ~Pool() override
+    {
+        {
+            std::lock_guard<std::mutex> lock(mu_);
+            stop_ = true;
+        }
+        wake_.notify_all();
+        for (auto& t : workers_) t.join();
+    }
+    int width() const override { return width_; }
+
+    void run(int pieces, const std::function<void(int)>& fn) override
+    {
+        if (pieces <= 0) return;
+        if (pieces == 1 || width_ == 1) {
+            for (int i = 0; i < pieces; ++i) fn(i);
+            return;
+        }
+        std::lock_guard<std::mutex> turn(job_mu_);  // one job at a time
+        uint64_t gen;
+        {
+            std::lock_guard<std::mutex> lock(mu_);
+            fn_ = &fn;
+            pieces_ = pieces;
+            next_ = 0;
+            left_ = pieces;
+            gen = ++generation_;
+        }
+        wake_.notify_all();
+        work(gen);  // the caller takes pieces too
+        std::unique_lock<std::mutex> lock(mu_);
+        done_.wait(lock, [this] { return left_ == 0; });
+        fn_ = nullptr;
+    }
+
+private:
+    // Takes pieces of job `gen` until none are left.  Pieces are handed out under the mutex (a job has at most
+    // `width` of them), so a thread that is late for its job can never take a piece of the next one by mistake.
+    void work(uint64_t gen)
+    {
+        for (;;) {
+            int i;
+            const std::function<void(int)>* fn;
+            {
+                std::lock_guard<std::mutex> lock(mu_);
+                if (gen != generation_ || next_ >= pieces_) return;
+                i = next_++;
+                fn = fn_;
+            }
+            (*fn)(i);
+            std::lock_guard<std::mutex> lock(mu_);
+            if (--left_ == 0) done_.notify_all();
+        }
+    }
+    void loop()
+    {
+        uint64_t seen = 0;
+        for (;;) {
+            {
+                std::unique_lock<std::mutex> lock(mu_);
+                wake_.wait(lock, [&] { return stop_ || generation_ != seen; });
+                if (stop_) return;
+                seen = generation_;
+            }
+            work(seen);
+        }
+    }
+
+    const int width_;
+    std::vector<std::thread> workers_;
+    std::mutex mu_, job_mu_;
+    std::condition_variable wake_, done_;
+    const std::function<void(int)>* fn_ = nullptr;
+    int pieces_ = 0, left_ = 0, next_ = 0;
+    uint64_t generation_ = 0;
+    bool stop_ = false;
+};
+
+int pool_width()
+{
+    int w = 8;
+    if (const char* e = getenv("PIMDL_COPY_THREADS")) w = atoi(e);
+    const int hw = (int)std::thread::hardware_concurrency();
+    if (hw > 0 && w > hw) w = hw;
+    if (w < 1) w = 1;
+    if (w > 64) w = 64;
+    return w;
+}
+
+}  // namespace
+
+HostPool& host_pool()
+{
+    static Pool pool(pool_width());
+    return pool;
+}
+
+void parallel_copy(void* dst, const void* src, size_t bytes)
+{
+    constexpr size_t SMALL = 256 * 1024;  // below this a hand-over to other threads costs more than it saves
+    HostPool& pool = host_pool();
+    if (bytes <= SMALL || pool.width() == 1) {
+        memcpy(dst, src, bytes);
+        return;
+    }
+    size_t pieces = (bytes + SMALL - 1) / SMALL;
+    if (pieces > (size_t)pool.width()) pieces = pool.width();
+    const size_t per = ((bytes + pieces - 1) / pieces + 63) & ~(size_t)63;
+    pool.run((int)pieces, [&](int i) {
+        const size_t off = (size_t)i * per;
+        if (off >= bytes) return;
+        const size_t len = off + per <= bytes ? per : bytes - off;
+        memcpy(static_cast<char*>(dst) + off, static_cast<const char*>(src) + off, len);
+    });
+}
+
+}  // namespace pimdl

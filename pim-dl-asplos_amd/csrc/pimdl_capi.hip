@@ -3,11 +3,19 @@
 // without a gfx950 device pimdl_init fails and nothing else can be called.
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
+#include <new>
+
+#include <algorithm>
+#include <chrono>
 #include <mutex>
+#include <set>
+#include <utility>
 #include <vector>
 
+#include "host_pool.h"
 #include "pimdl_internal.h"
 
 // Scratch of pimdl_amm_run_noalloc: the packed centroid indices that the search kernel writes and the gather
@@ -60,6 +68,18 @@ int hip_check(Ctx* ctx, hipError_t e, const char* what)
                      hipGetErrorString(e));
 }
 
+int allow_dynamic_lds(Ctx* ctx, const void* kernel, int lds_bytes, const char* what)
+{
+    static std::mutex mu;
+    static std::set<std::pair<int, const void*>> done;  // the attribute belongs to the kernel's code object on one device
+    std::lock_guard<std::mutex> lock(mu);
+    const std::pair<int, const void*> key(ctx->device, kernel);
+    if (done.count(key)) return PIMDL_OK;
+    int rc = hip_check(ctx, hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes), what);
+    if (!rc) done.insert(key);
+    return rc;
+}
+
 static bool is_device_ptr(const void* p)
 {
     hipPointerAttribute_t attr;
@@ -75,11 +95,14 @@ static bool is_device_ptr(const void* p)
 // Grow-only scratch.  A buffer that is too small is replaced by a larger one; the old one stays allocated until
 // the context is destroyed, because a HIP graph captured from earlier calls on this context holds its address
 // (both kernels of a captured AMM were given the same buffer, so a replay stays consistent with itself).
+// A buffer that grows does so by at least half its size, so that a caller whose batch creeps upwards goes through
+// a geometric series of buffers: the retired ones together stay below twice the size of the live one.
 // While the stream is being captured nothing may be allocated: the call is refused instead.
 template <typename T>
 static int ensure(Ctx* ctx, T** buf, size_t* have, size_t need, const char* what)
 {
     if (*have >= need) return PIMDL_OK;
+    if (*have && need < *have + *have / 2) need = *have + *have / 2;
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(ctx->stream, &cap) != hipSuccess) (void)hipGetLastError();
     if (cap != hipStreamCaptureStatusNone)
@@ -146,6 +169,179 @@ static int finish_output(Ctx* ctx, const AmmGeom& g, float* out, uint32_t n, boo
                                            ctx->stream), "D2H output");
     if (rc) return rc;
     return hip_check(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+}
+
+// ---- host buffers: the pinned staging ring ------------------------------------------------------------------
+// The reference's amm_host takes and returns ordinary (pageable) host memory.  A transfer straight from such
+// memory goes through the runtime's own single-threaded staging at about a fifth of the link's rate, so the
+// library stages by itself: the batch is cut into chunks of tokens (rows are independent), each chunk is copied
+// into a pinned buffer by the host thread pool, sent, searched and gathered on its own, sent back and copied out,
+// with HostPipe::SLOTS chunks in flight on three streams of equal priority.
+static void pipe_destroy(Ctx* ctx)
+{
+    HostPipe* hp = ctx->pipe;
+    if (!hp) return;
+    if (hp->s_in) (void)hipStreamSynchronize(hp->s_in);
+    if (hp->s_out) (void)hipStreamSynchronize(hp->s_out);
+    for (int s = 0; s < HostPipe::SLOTS; ++s) {
+        if (hp->pin_in[s]) (void)hipHostFree(hp->pin_in[s]);
+        if (hp->pin_out[s]) (void)hipHostFree(hp->pin_out[s]);
+        (void)hipFree(hp->d_in[s]);
+        (void)hipFree(hp->d_out[s]);
+        if (hp->ev_in[s]) (void)hipEventDestroy(hp->ev_in[s]);
+        if (hp->ev_run[s]) (void)hipEventDestroy(hp->ev_run[s]);
+        if (hp->ev_out[s]) (void)hipEventDestroy(hp->ev_out[s]);
+    }
+    if (hp->s_in) (void)hipStreamDestroy(hp->s_in);
+    if (hp->s_out) (void)hipStreamDestroy(hp->s_out);
+    delete hp;
+    ctx->pipe = nullptr;
+}
+
+static int pipe_get(Ctx* ctx, HostPipe** out)
+{
+    if (!ctx->pipe) {
+        HostPipe* hp = new (std::nothrow) HostPipe();
+        if (!hp) return set_error(ctx, PIMDL_ERR_NOMEM, "host staging: out of host memory");
+        ctx->pipe = hp;
+        int rc = hip_check(ctx, hipStreamCreateWithFlags(&hp->s_in, hipStreamNonBlocking), "hipStreamCreate(staging in)");
+        if (!rc) rc = hip_check(ctx, hipStreamCreateWithFlags(&hp->s_out, hipStreamNonBlocking), "hipStreamCreate(staging out)");
+        for (int s = 0; s < HostPipe::SLOTS && !rc; ++s) {
+            rc = hip_check(ctx, hipEventCreateWithFlags(&hp->ev_in[s], hipEventDisableTiming), "hipEventCreate");
+            if (!rc) rc = hip_check(ctx, hipEventCreateWithFlags(&hp->ev_run[s], hipEventDisableTiming), "hipEventCreate");
+            if (!rc) rc = hip_check(ctx, hipEventCreateWithFlags(&hp->ev_out[s], hipEventDisableTiming), "hipEventCreate");
+        }
+        if (rc) {
+            pipe_destroy(ctx);
+            return rc;
+        }
+    }
+    *out = ctx->pipe;
+    return PIMDL_OK;
+}
+
+// Per-slot buffers of at least the given sizes (0: that direction is not staged).  Only called while the ring is
+// idle (every call that uses it drains it before it returns or before it touches a slot again).
+static int pipe_reserve(Ctx* ctx, HostPipe* hp, size_t in_bytes, size_t out_bytes)
+{
+    int rc = PIMDL_OK;
+    if (in_bytes > hp->in_bytes) {
+        if ((rc = hip_check(ctx, hipStreamSynchronize(hp->s_in), "hipStreamSynchronize(staging in)"))) return rc;
+        if ((rc = hip_check(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"))) return rc;
+        for (int s = 0; s < HostPipe::SLOTS; ++s) {
+            if (hp->pin_in[s]) (void)hipHostFree(hp->pin_in[s]);
+            (void)hipFree(hp->d_in[s]);
+            hp->pin_in[s] = nullptr;
+            hp->d_in[s] = nullptr;
+        }
+        hp->in_bytes = 0;
+        for (int s = 0; s < HostPipe::SLOTS && !rc; ++s) {
+            rc = hip_check(ctx, hipHostMalloc(&hp->pin_in[s], in_bytes, hipHostMallocDefault), "hipHostMalloc(staging in)");
+            if (!rc) rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&hp->d_in[s]), in_bytes), "hipMalloc(staging in)");
+        }
+        if (rc) return rc;
+        hp->in_bytes = in_bytes;
+    }
+    if (out_bytes > hp->out_bytes) {
+        if ((rc = hip_check(ctx, hipStreamSynchronize(hp->s_out), "hipStreamSynchronize(staging out)"))) return rc;
+        if ((rc = hip_check(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"))) return rc;
+        for (int s = 0; s < HostPipe::SLOTS; ++s) {
+            if (hp->pin_out[s]) (void)hipHostFree(hp->pin_out[s]);
+            (void)hipFree(hp->d_out[s]);
+            hp->pin_out[s] = nullptr;
+            hp->d_out[s] = nullptr;
+        }
+        hp->out_bytes = 0;
+        for (int s = 0; s < HostPipe::SLOTS && !rc; ++s) {
+            rc = hip_check(ctx, hipHostMalloc(&hp->pin_out[s], out_bytes, hipHostMallocDefault), "hipHostMalloc(staging out)");
+            if (!rc) rc = hip_check(ctx, hipMalloc(reinterpret_cast<void**>(&hp->d_out[s]), out_bytes), "hipMalloc(staging out)");
+        }
+        if (rc) return rc;
+        hp->out_bytes = out_bytes;
+    }
+    return PIMDL_OK;
+}
+
+// tokens per chunk: about 6 MiB of the wider staged side, a multiple of 512 tokens (whole items of every gather)
+static uint32_t pipe_chunk_tokens(uint32_t n, size_t row_bytes)
+{
+    const char* e = getenv("PIMDL_HOST_CHUNK_TOKENS");
+    uint64_t t = e ? strtoull(e, nullptr, 10) : 0;
+    if (!t) t = (6u << 20) / (row_bytes ? row_bytes : 1);
+    t = t / 512 * 512;
+    if (t < 512) t = 512;
+    return t >= n ? n : (uint32_t)t;
+}
+
+// One AMM with at least one of in / out in host memory.  `run_chunk(d_in, d_out, tokens)` queues the kernels of
+// one chunk on the context's stream.  Synchronous when out is a host buffer; with a device `out` the call returns
+// once `in` has been copied to pinned memory (the caller may reuse it), the rest is ordered on the streams.
+template <class RunChunk>
+static int run_piped(Ctx* ctx, uint32_t K, uint32_t M, const float* in, bool in_host, float* out, bool out_host,
+                     uint32_t n, RunChunk run_chunk)
+{
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(ctx->stream, &cap) != hipSuccess) (void)hipGetLastError();
+    if (cap != hipStreamCaptureStatusNone)
+        return set_error(ctx, PIMDL_ERR_INVALID, "host buffers cannot be staged while the stream is being captured: pass device pointers");
+    HostPipe* hp;
+    int rc = pipe_get(ctx, &hp);
+    if (rc) return rc;
+    constexpr int SLOTS = HostPipe::SLOTS, LAG = SLOTS - 1;
+    const size_t in_row = (size_t)K * sizeof(float), out_row = (size_t)M * sizeof(float);
+    const size_t wide = (in_host ? in_row : 0) > (out_host ? out_row : 0) ? in_row : out_row;
+    const uint32_t chunk = pipe_chunk_tokens(n, wide);
+    const uint32_t nchunks = (n + chunk - 1) / chunk;
+    if ((rc = pipe_reserve(ctx, hp, in_host ? chunk * in_row : 0, out_host ? chunk * out_row : 0))) return rc;
+
+    auto fail = [&](int code) {  // nothing may stay in flight towards buffers the caller owns
+        (void)hipStreamSynchronize(hp->s_in);
+        (void)hipStreamSynchronize(ctx->stream);
+        (void)hipStreamSynchronize(hp->s_out);
+        return code;
+    };
+    auto tokens_of = [&](uint32_t c) { return c + 1 == nchunks ? n - c * chunk : chunk; };
+    for (uint32_t c = 0; c < nchunks + (out_host ? LAG : 0); ++c) {
+        if (c < nchunks) {
+            const int s = c % SLOTS;
+            const uint32_t tok = tokens_of(c);
+            const float* d_in = in + (size_t)c * chunk * K;
+            float* d_out = out + (size_t)c * chunk * M;
+            if (in_host) {
+                // the slot's pinned buffer is free once its last transfer has left it
+                if (hp->used_in[s] && (rc = hip_check(ctx, hipEventSynchronize(hp->ev_in[s]), "hipEventSynchronize(staging in)"))) return fail(rc);
+                parallel_copy(hp->pin_in[s], d_in, tok * in_row);
+                // ... and its device buffer once the kernels that read it are done
+                if (hp->used_run[s] && (rc = hip_check(ctx, hipStreamWaitEvent(hp->s_in, hp->ev_run[s], 0), "hipStreamWaitEvent"))) return fail(rc);
+                if ((rc = hip_check(ctx, hipMemcpyAsync(hp->d_in[s], hp->pin_in[s], tok * in_row, hipMemcpyHostToDevice, hp->s_in), "H2D input chunk"))) return fail(rc);
+                if ((rc = hip_check(ctx, hipEventRecord(hp->ev_in[s], hp->s_in), "hipEventRecord"))) return fail(rc);
+                hp->used_in[s] = true;
+                if ((rc = hip_check(ctx, hipStreamWaitEvent(ctx->stream, hp->ev_in[s], 0), "hipStreamWaitEvent"))) return fail(rc);
+                d_in = hp->d_in[s];
+            }
+            if (out_host) {
+                // the slot's device output is free once its last transfer back has read it
+                if (hp->used_out[s] && (rc = hip_check(ctx, hipStreamWaitEvent(ctx->stream, hp->ev_out[s], 0), "hipStreamWaitEvent"))) return fail(rc);
+                d_out = hp->d_out[s];
+            }
+            if ((rc = run_chunk(d_in, d_out, tok))) return fail(rc);
+            if ((rc = hip_check(ctx, hipEventRecord(hp->ev_run[s], ctx->stream), "hipEventRecord"))) return fail(rc);
+            hp->used_run[s] = true;
+            if (out_host) {
+                if ((rc = hip_check(ctx, hipStreamWaitEvent(hp->s_out, hp->ev_run[s], 0), "hipStreamWaitEvent"))) return fail(rc);
+                if ((rc = hip_check(ctx, hipMemcpyAsync(hp->pin_out[s], hp->d_out[s], tok * out_row, hipMemcpyDeviceToHost, hp->s_out), "D2H output chunk"))) return fail(rc);
+                if ((rc = hip_check(ctx, hipEventRecord(hp->ev_out[s], hp->s_out), "hipEventRecord"))) return fail(rc);
+                hp->used_out[s] = true;
+            }
+        }
+        if (out_host && c >= (uint32_t)LAG) {  // chunk c - LAG has had LAG iterations to come back
+            const uint32_t r = c - LAG;
+            const int s = r % SLOTS;
+            if ((rc = hip_check(ctx, hipEventSynchronize(hp->ev_out[s]), "hipEventSynchronize(staging out)"))) return fail(rc);
+            parallel_copy(out + (size_t)r * chunk * M, hp->pin_out[s], tokens_of(r) * out_row);
+        }
+    }
+    return PIMDL_OK;
 }
 
 static int check_run_args(Amm* amm, const void* a, const void* b, uint32_t n)
@@ -250,13 +446,15 @@ int pimdl_init(int device, pimdl_ctx** out)
     ctx->d_tmp = nullptr; ctx->tmp_bytes = 0;
     ctx->d_cent = nullptr; ctx->cent_bytes = 0;
     ctx->d_static_scratch = nullptr;
+    ctx->pipe = nullptr;
     for (auto& ev : ctx->ev) ev = nullptr;
     int rc = hip_check(ctx, hipSetDevice(device), "hipSetDevice");
-    if (!rc) rc = static_scratch_address(ctx, device, &ctx->d_static_scratch);
     if (!rc) rc = hip_check(ctx, hipGetDeviceProperties(&ctx->prop, device), "hipGetDeviceProperties");
     if (!rc && strncmp(ctx->prop.gcnArchName, "gfx950", 6) != 0)
         rc = set_error(ctx, PIMDL_ERR_UNSUPPORTED, "pimdl_init: device %d is %s; the kernels are built for gfx950 only",
                        device, ctx->prop.gcnArchName);
+    // (after the check above: on another device the library's code object, and with it the symbol, does not exist)
+    if (!rc) rc = static_scratch_address(ctx, device, &ctx->d_static_scratch);
     if (!rc) rc = hip_check(ctx, hipStreamCreate(&ctx->own_stream), "hipStreamCreate");
     for (auto& ev : ctx->ev)
         if (!rc) rc = hip_check(ctx, hipEventCreate(&ev), "hipEventCreate");
@@ -275,6 +473,7 @@ int pimdl_destroy(pimdl_ctx* ctx)
     if (!ctx) return PIMDL_OK;
     (void)hipSetDevice(ctx->device);
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    pipe_destroy(ctx);
     (void)hipFree(ctx->d_in);
     (void)hipFree(ctx->d_out);
     (void)hipFree(ctx->d_idx);
@@ -439,9 +638,14 @@ int pimdl_amm_create_with(pimdl_ctx* ctx, const pimdl_amm_desc* desc, const floa
     if (!rc) rc = launch_ccs_prep(ctx, g, a->d_centroids);
     if (!rc) rc = hip_check(ctx, hipMemcpy(a->d_lut, tiled.data(), a->lut_bytes, hipMemcpyHostToDevice), "H2D lut");
     if (!rc) {
-        if (bias) rc = hip_check(ctx, hipMemcpy(a->d_bias, bias, (size_t)g.M * sizeof(float), hipMemcpyHostToDevice), "H2D bias");
-        else rc = hip_check(ctx, hipMemset(a->d_bias, 0, (size_t)g.M * sizeof(float)), "memset bias");
+        try {
+            if (bias) a->h_bias.assign(bias, bias + g.M);
+            else a->h_bias.assign(g.M, 0.0f);
+        } catch (...) {
+            rc = set_error(ctx, PIMDL_ERR_NOMEM, "pimdl_amm_create: out of host memory");
+        }
     }
+    if (!rc) rc = hip_check(ctx, hipMemcpy(a->d_bias, a->h_bias.data(), (size_t)g.M * sizeof(float), hipMemcpyHostToDevice), "H2D bias");
     if (!rc && a->nscales) rc = hip_check(ctx, hipMemcpy(a->d_scales, scales, sizeof(float) * a->nscales, hipMemcpyHostToDevice), "H2D scales");
     // the index scratch of the largest batch now, so that runs on device buffers never allocate
     if (!rc) rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, idx_buffer_bytes(g, desc->max_n), "hipMalloc(index scratch)");
@@ -460,11 +664,29 @@ int pimdl_amm_set_bias(pimdl_amm* a, const float* bias)
     int rc = activate(ctx);
     if (rc) return rc;
     const size_t bytes = (size_t)a->g.M * sizeof(float);
+    // the device already holds these values: nothing to send, nothing to wait for
+    if (a->h_bias.size() == a->g.M &&
+        (bias ? memcmp(a->h_bias.data(), bias, bytes) == 0
+              : std::all_of(a->h_bias.begin(), a->h_bias.end(), [](float f) { uint32_t b; memcpy(&b, &f, 4); return b == 0; })))
+        return PIMDL_OK;
+    // a copy and a wait cannot be recorded into a graph
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(ctx->stream, &cap) != hipSuccess) (void)hipGetLastError();
+    if (cap != hipStreamCaptureStatusNone)
+        return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_set_bias: the stream is being captured; change the bias outside the capture");
+    try {
+        if (bias) a->h_bias.assign(bias, bias + a->g.M);
+        else a->h_bias.assign(a->g.M, 0.0f);
+    } catch (...) {
+        return set_error(ctx, PIMDL_ERR_NOMEM, "pimdl_amm_set_bias: out of host memory");
+    }
     // ordered on the context's stream behind the launches that still read the old values
-    if (bias) rc = hip_check(ctx, hipMemcpyAsync(a->d_bias, bias, bytes, hipMemcpyHostToDevice, ctx->stream), "H2D bias");
-    else rc = hip_check(ctx, hipMemsetAsync(a->d_bias, 0, bytes, ctx->stream), "clear bias");
-    if (rc) return rc;
-    return hip_check(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");  // `bias` may be reused on return
+    rc = hip_check(ctx, hipMemcpyAsync(a->d_bias, a->h_bias.data(), bytes, hipMemcpyHostToDevice, ctx->stream), "H2D bias");
+    if (rc) {
+        a->h_bias.clear();
+        return rc;
+    }
+    return hip_check(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
 }
 
 int pimdl_amm_destroy(pimdl_amm* a)
@@ -650,15 +872,14 @@ int pimdl_amm_run(pimdl_amm* a, const float* in, uint32_t n, float* out)
     int rc = check_run_args(a, in, out, n);
     if (rc || n == 0) return rc;
     Ctx* ctx = a->ctx;
-    const float* d_in;
-    float* d_out;
-    bool out_host;
-    if ((rc = stage_input(ctx, a->g, in, n, &d_in))) return rc;
-    if ((rc = stage_output(ctx, a->g, out, n, &d_out, &out_host))) return rc;
     if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, idx_buffer_bytes(a->g, n), "hipMalloc(index scratch)"))) return rc;
-    if ((rc = launch_ccs(ctx, a->g, d_in, a->d_centroids, ctx->d_idx, n))) return rc;
-    if ((rc = launch_gather(ctx, *a, ctx->d_idx, d_out, nullptr, n))) return rc;
-    return finish_output(ctx, a->g, out, n, out_host);
+    auto run_rows = [&](const float* d_in, float* d_out, uint32_t tokens) -> int {
+        int r = launch_ccs(ctx, a->g, d_in, a->d_centroids, ctx->d_idx, tokens);
+        return r ? r : launch_gather(ctx, *a, ctx->d_idx, d_out, nullptr, tokens);
+    };
+    const bool in_host = !is_device_ptr(in), out_host = !is_device_ptr(out);
+    if (in_host || out_host) return run_piped(ctx, a->g.K, a->g.M, in, in_host, out, out_host, n, run_rows);
+    return run_rows(in, out, n);
 }
 
 int pimdl_amm_run_noalloc(pimdl_amm* a, const float* in_dev, uint32_t n, float* out_dev)
@@ -835,11 +1056,56 @@ int pimdl_amm_run_tiled(pimdl_amm* a, const float* in, uint32_t n, float* out, c
     pimdl_tiling til;
     bool ident;
     if ((rc = resolve_tiling(ctx, a->g, n, tiling, &til, &ident))) return rc;
+    if (ident) return pimdl_amm_run(a, in, n, out);  // row-major in and out (the search never sees cb_mtile_size)
     const float* d_in;
     if ((rc = stage_input(ctx, a->g, in, n, &d_in))) return rc;
     if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, idx_buffer_bytes(a->g, n), "hipMalloc(index scratch)"))) return rc;
     if ((rc = launch_ccs(ctx, a->g, d_in, a->d_centroids, ctx->d_idx, n))) return rc;
     return gather_to(a, n, out, til, ident);
+}
+
+int pimdl_amm_run_breakdown(pimdl_amm* a, const float* in, uint32_t n, float* out, const pimdl_tiling* tiling,
+                            pimdl_amm_breakdown* acc)
+{
+    int rc = check_run_args(a, in, out, n);
+    if (rc) return rc;
+    Ctx* ctx = a->ctx;
+    if (!acc) return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_amm_run_breakdown: null result pointer");
+    if (n == 0) return PIMDL_OK;
+    pimdl_tiling til;
+    bool ident;
+    if ((rc = resolve_tiling(ctx, a->g, n, tiling, &til, &ident))) return rc;
+    auto now = [] { return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count(); };
+    auto sync = [&] { return hip_check(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize"); };
+    // one phase after the other, each waited for, as the reference's own breakdown does (dpu_sync between phases)
+    if ((rc = sync())) return rc;
+    const double t0 = now();
+    const float* d_in;
+    if ((rc = stage_input(ctx, a->g, in, n, &d_in))) return rc;
+    if ((rc = ensure(ctx, &ctx->d_idx, &ctx->idx_bytes, idx_buffer_bytes(a->g, n), "hipMalloc(index scratch)"))) return rc;
+    float* d_out;
+    bool out_host;
+    if ((rc = stage_output(ctx, a->g, out, n, &d_out, &out_host))) return rc;
+    if (!ident && (rc = ensure(ctx, &ctx->d_tmp, &ctx->tmp_bytes, (size_t)n * a->g.M * 4, "hipMalloc(row-major scratch)"))) return rc;
+    if ((rc = sync())) return rc;
+    const double t1 = now();
+    if ((rc = launch_ccs(ctx, a->g, d_in, a->d_centroids, ctx->d_idx, n))) return rc;
+    if ((rc = sync())) return rc;
+    const double t2 = now();
+    if ((rc = launch_gather(ctx, *a, ctx->d_idx, ident ? d_out : ctx->d_tmp, nullptr, n))) return rc;
+    if (!ident && (rc = launch_retile_output(ctx, ctx->d_tmp, d_out, n, a->g.M, til.n_stile_size, til.feature_stile_size,
+                                             til.feature_mtile_size)))
+        return rc;
+    if ((rc = sync())) return rc;
+    const double t3 = now();
+    if ((rc = finish_output(ctx, a->g, out, n, out_host))) return rc;
+    if ((rc = sync())) return rc;
+    const double t4 = now();
+    acc->h2d_s += t1 - t0;
+    acc->search_s += t2 - t1;
+    acc->gather_s += t3 - t2;
+    acc->d2h_s += t4 - t3;
+    return PIMDL_OK;
 }
 
 int pimdl_lut_gather_tiled(pimdl_amm* a, const uint16_t* idx, uint32_t n, float* out, const pimdl_tiling* tiling)

@@ -77,6 +77,7 @@ struct Amm {
     float* d_scales;     // int8: scales
     uint32_t nscales;
     float* d_bias;       // [M]
+    std::vector<float> h_bias;  // what d_bias holds (pimdl_amm_set_bias skips the copy when nothing changed)
     float h_scale0;
     bool grouped;        // int8 LUT with scale_group > 0: resident as fp32 integers, fp32 gather kernel
     bool prescaled;      // ... with scale_group == 1: resident already multiplied by its codebook's scale (the one
@@ -95,6 +96,21 @@ struct Amm {
         last_tokens_per_wg = tokens_per_wg;
         last_threads = threads;
     }
+};
+
+// Pinned staging ring of the host-buffer path (pimdl_capi.hip): SLOTS chunks of tokens in flight, each with a
+// pinned and a device buffer per direction, so that the caller's copy into pinned memory, the transfer to the
+// device, the two kernels, the transfer back and the copy out of pinned memory of different chunks overlap.
+struct HostPipe {
+    static constexpr int SLOTS = 4;
+    hipStream_t s_in = nullptr, s_out = nullptr;       // transfers; the kernels run on the context's stream
+    hipEvent_t ev_in[SLOTS] = {}, ev_run[SLOTS] = {}, ev_out[SLOTS] = {};
+    bool used_in[SLOTS] = {}, used_run[SLOTS] = {}, used_out[SLOTS] = {};  // the event has been recorded at least once
+    void* pin_in[SLOTS] = {};
+    void* pin_out[SLOTS] = {};
+    float* d_in[SLOTS] = {};
+    float* d_out[SLOTS] = {};
+    size_t in_bytes = 0, out_bytes = 0;                // per slot
 };
 
 struct Ctx {
@@ -122,10 +138,13 @@ struct Ctx {
     float* d_cent;       // centroids of a context-level pimdl_index_calculation call
     size_t cent_bytes;
     hipEvent_t ev[4];
+    HostPipe* pipe;      // created by the first call that hands over a host buffer
 };
 
 int set_error(Ctx* ctx, int code, const char* fmt, ...);
 int hip_check(Ctx* ctx, hipError_t e, const char* what);
+// Raises a kernel's dynamic LDS limit to `lds_bytes`, once per (device of ctx, kernel); safe from several threads.
+int allow_dynamic_lds(Ctx* ctx, const void* kernel, int lds_bytes, const char* what);
 
 // kernels (launchers validate nothing: callers have already checked shapes against AmmGeom)
 // x_cols != 0: the geometry's codebooks are those of several operators that all read rows of x_cols

@@ -2,8 +2,14 @@
 // (what `python run_amm.py --amm_config_file X.yaml` ends up running).
 //
 //   test_amm <kernel_config.yaml> [dpu_binary_path (ignored)] [--dump FILE] [--rounds WARMUP RECORD]
-//            [--split] [--load-type 0|1|2] [--refill]
+//            [--split] [--load-type 0|1|2] [--refill] [--breakdown] [--assume-unchanged]
 //
+//   --breakdown  every amm_host call prints the two lines of the reference's AMM_BREAKDOWN build, cumulative seconds:
+//                "index calculation time" (amm_host.cpp:24) and "other latency ..., data transfer latency ..., pim
+//                kernel latency ..." (pim_lut_host.cpp:211); the phases then run one after the other
+//   --assume-unchanged  skip the per-call hash of LUT and centroids (PimdlHostOptions::assume_unchanged); with
+//                --refill the in-place changes of LUT and centroids then go unnoticed (the bias is still compared on
+//                every call), and the dump holds the LUT and the centroids as they were uploaded
 //   --split      every round calls index_calculation() and then pim_lut() (the two halves amm_host is made of,
 //                amm_host.cpp:10-30) instead of amm_host(); the dump then also holds the index buffer as
 //                pim_lut leaves it (rewritten in place, pim_lut_host.cpp:40-104)
@@ -167,7 +173,7 @@ int main(int argc, char** argv)
 {
     if (argc < 2) {
         printf("usage: %s kernel_config_yaml_path [dpu_binary_path] [--dump FILE] [--rounds WARMUP RECORD] [--split] "
-               "[--load-type T] [--refill]\n", argv[0]);
+               "[--load-type T] [--refill] [--breakdown] [--assume-unchanged]\n", argv[0]);
         return -1;
     }
     string dump_path;
@@ -178,6 +184,8 @@ int main(int argc, char** argv)
         if (!strcmp(argv[i], "--dump") && i + 1 < argc) dump_path = argv[++i];
         else if (!strcmp(argv[i], "--split")) split = true;
         else if (!strcmp(argv[i], "--refill")) refill = true;
+        else if (!strcmp(argv[i], "--breakdown")) pimdl_host_options().breakdown = true;
+        else if (!strcmp(argv[i], "--assume-unchanged")) pimdl_host_options().assume_unchanged = true;
         else if (!strcmp(argv[i], "--load-type") && i + 1 < argc) load_type = atoi(argv[++i]);
         else if (!strcmp(argv[i], "--rounds") && i + 2 < argc) {
             warmup = atoi(argv[++i]);
@@ -227,6 +235,9 @@ int main(int argc, char** argv)
     load_binary(&dpu_set, argc > 2 && argv[2][0] != '-' ? argv[2] : "");
     cout << "binary load time is " << now_s() - t1 << endl;
 
+    const bool assume_unchanged = pimdl_host_options().assume_unchanged;
+    const vector<lut_data_type> uploaded_lut = assume_unchanged ? cpu_lut : vector<lut_data_type>();
+    const vector<float> uploaded_centroids = assume_unchanged ? centroids : vector<float>();
     vector<index_data_type> index_buffer(split ? (size_t)ip.n * ip.num_codebook : 0);
     double total = 0.0;
     for (int round = 0; round < warmup + record; ++round) {
@@ -271,8 +282,8 @@ int main(int argc, char** argv)
         fwrite(&lp.scale, 4, 1, fp);
         fwrite(&lp.bias, 4, 1, fp);
         fwrite(input.data(), 4, input.size(), fp);
-        fwrite(centroids.data(), 4, centroids.size(), fp);
-        fwrite(cpu_lut.data(), 1, cpu_lut.size(), fp);
+        fwrite(assume_unchanged ? uploaded_centroids.data() : centroids.data(), 4, centroids.size(), fp);
+        fwrite(assume_unchanged ? uploaded_lut.data() : cpu_lut.data(), 1, cpu_lut.size(), fp);
         fwrite(bias.data(), 4, bias.size(), fp);
         fwrite(output.data(), 4, output.size(), fp);
         if (split) fwrite(index_buffer.data(), sizeof(index_data_type), index_buffer.size(), fp);

@@ -110,6 +110,114 @@ def test_inputs_changed_in_place_between_calls(tmp_path, flags):
     assert np.array_equal(d["out"].view(np.uint32), expected_tiled_output(d).view(np.uint32))
 
 
+def test_assume_unchanged_skips_the_change_detection(tmp_path):
+    """PimdlHostOptions::assume_unchanged: LUT and centroids are not read again once uploaded, so their in-place
+    changes before the last call go unnoticed (the dump then holds them as uploaded), while the bias tensor, which
+    is compared on every call, is followed.  Without changes the option changes nothing."""
+    stdout, d = run_cli(tmp_path, "--assume-unchanged", "--rounds", "1", "2")
+    assert np.array_equal(d["out"].view(np.uint32), expected_tiled_output(d).view(np.uint32))
+    stdout, d = run_cli(tmp_path, "--assume-unchanged", "--refill", "--rounds", "1", "2")
+    assert "inputs changed in place" in stdout
+    assert np.array_equal(d["out"].view(np.uint32), expected_tiled_output(d).view(np.uint32))
+    # the same run without the option sees the new tables: another output
+    _, d2 = run_cli(tmp_path, "--refill", "--rounds", "1", "2")
+    assert np.array_equal(d2["bias"], d["bias"]) and not np.array_equal(d2["lut"], d["lut"])
+    assert not np.array_equal(d2["out"], d["out"])
+
+
+def test_breakdown_lines_of_the_reference(tmp_path):
+    """--breakdown: the two lines the reference's AMM_BREAKDOWN build prints per call (amm_host.cpp:24,
+    pim_lut_host.cpp:211), cumulative seconds that only grow, and the same output bits."""
+    import re
+    stdout, d = run_cli(tmp_path, "--breakdown", "--rounds", "1", "3")
+    assert np.array_equal(d["out"].view(np.uint32), expected_tiled_output(d).view(np.uint32))
+    ic = [float(m) for m in re.findall(r"^index calculation time (\d+\.\d{6})$", stdout, re.M)]
+    rest = re.findall(r"^other latency (\d+\.\d{6}), data transfer latency (\d+\.\d{6}), pim kernel latency (\d+\.\d{6})$", stdout, re.M)
+    assert len(ic) == 4 and len(rest) == 4
+    cols = np.array([[float(v) for v in r] for r in rest])
+    assert all(np.diff(ic) > 0) and (np.diff(cols, axis=0) >= 0).all() and (cols[-1] > 0).all()
+
+
+def test_host_buffers_in_chunks(ctx, monkeypatch):
+    """Host pointers go through the pinned staging ring in chunks of tokens; with 512-token chunks a batch of 3000
+    tokens is six chunks, the last one ragged, on four slots.  Every combination of host and device buffers gives
+    the bits of one launch over the whole batch on device buffers (and those are the oracle's)."""
+    import torch
+    monkeypatch.setenv("PIMDL_HOST_CHUNK_TOKENS", "512")
+    rng = np.random.default_rng(31)
+    N, K, v, C, M = 3000, 256, 4, 16, 320
+    CB = K // v
+    x = rng.standard_normal((N, K)).astype(np.float32)
+    cent = rng.standard_normal((CB, C, v)).astype(np.float32)
+    lut = rng.integers(-128, 128, (CB, C, M)).astype(np.int8)
+    bias = rng.standard_normal(M).astype(np.float32)
+    amm = ctx.amm(cent, lut, np.float32(0.05), bias, max_n=N)
+    want, _, _ = oracle.amm_cpu(x, cent, lut, bias, v, 0.05, 0.0, threads=THREADS)
+    xd = torch.from_numpy(x).cuda()
+    yd = torch.zeros((N, M), device="cuda")
+    amm.run_ptr(xd.data_ptr(), N, yd.data_ptr())
+    ctx.synchronize()
+    assert np.array_equal(yd.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    for n in (N, 512, 513, 1):
+        # host -> host
+        out = np.full((n, M), -7.0, np.float32)
+        amm.run_ptr(x.ctypes.data, n, out.ctypes.data)
+        assert np.array_equal(out.view(np.uint32), want[:n].view(np.uint32)), n
+        # host -> device (returns once the input is copied; the rest is stream-ordered)
+        yd.fill_(-7.0)
+        torch.cuda.synchronize()
+        xcopy = x[:n].copy()
+        amm.run_ptr(xcopy.ctypes.data, n, yd.data_ptr())
+        xcopy[:] = 0.0   # the caller may reuse its input
+        ctx.synchronize()
+        assert np.array_equal(yd[:n].cpu().numpy().view(np.uint32), want[:n].view(np.uint32)), n
+        # device -> host
+        out = np.full((n, M), -7.0, np.float32)
+        amm.run_ptr(xd.data_ptr(), n, out.ctypes.data)
+        assert np.array_equal(out.view(np.uint32), want[:n].view(np.uint32)), n
+    # a second operator with wider rows makes the ring's buffers grow
+    M2 = 1024
+    lut2 = rng.integers(-128, 128, (CB, C, M2)).astype(np.int8)
+    amm2 = ctx.amm(cent, lut2, np.float32(0.05), None, max_n=N)
+    want2, _, _ = oracle.amm_cpu(x, cent, lut2, np.zeros(M2, np.float32), v, 0.05, 0.0, threads=THREADS)
+    out2 = np.empty((N, M2), np.float32)
+    amm2.run_ptr(x.ctypes.data, N, out2.ctypes.data)
+    assert np.array_equal(out2.view(np.uint32), want2.view(np.uint32))
+    out = np.empty((N, M), np.float32)
+    amm.run_ptr(x.ctypes.data, N, out.ctypes.data)
+    assert np.array_equal(out.view(np.uint32), want.view(np.uint32))
+    amm.close()
+    amm2.close()
+
+
+def test_scratch_of_a_creeping_batch_stays_bounded():
+    """A caller whose batch grows call by call: the context's grow-only scratch is replaced by geometrically larger
+    buffers (old ones are kept for HIP graphs that may hold them), so what it holds in the end is a small multiple
+    of what the largest call needs, not the sum over all calls."""
+    import torch
+    c = pimdl.Context(0)
+    rng = np.random.default_rng(32)
+    K, v, C, M = 64, 4, 16, 512
+    CB = K // v
+    cent = rng.standard_normal((CB, C, v)).astype(np.float32)
+    lut = rng.integers(-128, 128, (CB, C, M)).astype(np.int8)
+    x = rng.standard_normal((2000, K)).astype(np.float32)
+    amm = c.amm(cent, lut, np.float32(1.0), None, max_n=2000)
+    amm.run_debug(x[:1])           # the debug path stages through the grow-only scratch (output, accumulators, ids)
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    for n in range(2, 2001, 3):
+        amm.run_debug(x[:n])
+    torch.cuda.synchronize()
+    grown = free0 - torch.cuda.mem_get_info()[0]
+    # the last call needs 2000 x (512 x 4 out + 512 x 4 acc + 16 x 2 ids + 64 x 4 in) = 8.8 MB; exact-size growth with
+    # the old buffers kept would hold the sum over 667 calls, about 3 GB (the bound leaves room for the allocator's
+    # own granularity on some eighty small buffers)
+    assert grown < 256 << 20, grown
+    amm.close()
+    c.close()
+
+
 def test_index_ids_out_of_range_are_refused(ctx):
     rng = np.random.default_rng(5)
     N, CB, C, M = 40, 6, 12, 32

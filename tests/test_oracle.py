@@ -334,6 +334,30 @@ def test_layout_helpers():
     assert np.array_equal(oracle.prepare_input_index(idx, N, CB, C, N, CB, 2, 24, 8, 2).reshape(N, CB), want)
 
 
+@pytest.mark.parametrize("N,CB,C,ns,cm,fs,flt,cblt", [(12, 8, 16, 4, 4, 24, 8, 2), (6, 12, 5, 3, 6, 10, 5, 3),
+                                                      (8, 8, 32, 2, 8, 4096, 4096, 4)])
+def test_prepare_input_index_under_a_dpu_tiling(N, CB, C, ns, cm, fs, flt, cblt):
+    """pim_lut_host.cpp:40-104 on a buffer in the search's tiled order (index_calc_host.cpp:41-49), stated without
+    the offset formula: that order is the row-major [N][CB] array cut into (N/ns, ns, CB/cm, cm) with the two middle
+    axes swapped, and the rewrite depends on an entry's value and on its position inside its cb_mtile only.  The
+    last case overflows 16 bits, which the reference's uint16 buffer truncates."""
+    rng = np.random.default_rng(N * 131 + CB)
+    idx = rng.integers(0, C, (N, CB)).astype(np.uint16)
+    tiled = np.ascontiguousarray(idx.reshape(N // ns, ns, CB // cm, cm).transpose(0, 2, 1, 3))   # [n_tile][cb_tile][n_in][cb_in]
+    wide = tiled.astype(np.uint32)
+    cb_in = np.arange(cm, dtype=np.uint32)[None, None, None, :]
+    want = {0: wide * fs, 1: wide * flt, 2: (cb_in % cblt) * C * flt + wide * flt}
+    for load_type in (0, 1, 2):
+        got = oracle.prepare_input_index(tiled.reshape(-1), N, CB, C, ns, cm, load_type, fs, flt, cblt)
+        assert np.array_equal(got.reshape(tiled.shape), (want[load_type] & 0xFFFF).astype(np.uint16)), load_type
+    # the search's own tiled output is that same array view (ties the two layout statements together)
+    x = rng.standard_normal((N, CB * 2)).astype(np.float32)
+    cent = rng.standard_normal((CB, C, 2)).astype(np.float32)
+    rm = oracle.index_calculation(x, cent, 2)
+    til = oracle.index_calculation(x, cent, 2, n_stile=ns, cb_mtile=cm)
+    assert np.array_equal(np.asarray(til).reshape(N // ns, CB // cm, ns, cm), rm.reshape(N // ns, ns, CB // cm, cm).transpose(0, 2, 1, 3))
+
+
 def test_layer_norm_closed_form():
     rng = np.random.default_rng(20)
     x = rng.standard_normal((6, 64)).astype(np.float32) * 3 + 1

@@ -73,7 +73,8 @@ def test_noalloc_matches_run_on_two_calls_in_a_row(ctx):
     assert np.array_equal(got2.view(np.uint32), want2.view(np.uint32))
     amm.close()
 
-    # another operator on the same array: 8-bit indices (32 centroids, the byte-adder gather), fewer codebooks
+    # another operator on the same array: 8-bit indices (32 centroids: one byte per codebook in the tiled order
+    # of the matrix-core gather), fewer codebooks
     N3, K3, v3, C3, M3 = 77, 96, 8, 32, 100
     x3, cent3, lut3, bias3 = _case(12, N3, K3, v3, C3, M3)
     amm3 = ctx.amm(cent3, lut3, np.float32(0.5), bias3, max_n=N3)
@@ -83,6 +84,53 @@ def test_noalloc_matches_run_on_two_calls_in_a_row(ctx):
     want3 = oracle.dequant(oracle.gather_i8(idx3, lut3, threads=THREADS), bias3, K3 // v3, 0.5, 0.0, 0, threads=THREADS)
     assert np.array_equal(got3.view(np.uint32), want3.view(np.uint32))
     amm3.close()
+
+
+def test_noalloc_first_call_on_a_fresh_context_allocates_nothing():
+    """The entry point on a context and operator that have never seen pimdl_amm_run (nothing has sized the
+    context's scratch buffers for it), with 64 centroids: row-major index rows of one byte per codebook and the
+    byte-adder gather go through the fixed array.  Device memory in use must not change across the calls."""
+    import torch
+
+    N, K, v, C, M = 500, 256, 4, 64, 128
+    x, cent, lut, bias = _case(15, N, K, v, C, M)
+    idx = oracle.index_calculation(x, cent, v, threads=THREADS)
+    want = oracle.dequant(oracle.gather_i8(idx, lut, threads=THREADS), bias, K // v, 0.25, 0.0, 0, threads=THREADS)
+    xd = torch.from_numpy(x).cuda()
+    got1 = torch.full((N, M), -5.0, device="cuda")
+    got2 = torch.full((200, M), -5.0, device="cuda")
+    # the kernels' code objects reach the device at their first launch: take that out of the measurement with
+    # the same entry point on another context
+    warm = pimdl.Context(0)
+    wamm = warm.amm(cent, lut, np.float32(0.25), bias, max_n=N)
+    wamm.run_noalloc_ptr(xd.data_ptr(), N, got1.data_ptr())
+    warm.synchronize()
+    got1.fill_(-5.0)
+
+    fresh = pimdl.Context(0)
+    amm = fresh.amm(cent, lut, np.float32(0.25), bias, max_n=N)
+    assert amm.last_gather_kernel() == ""   # never launched
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    amm.run_noalloc_ptr(xd.data_ptr(), N, got1.data_ptr())
+    fresh.synchronize()
+    free1 = torch.cuda.mem_get_info()[0]
+    amm.run_noalloc_ptr(xd.data_ptr(), 200, got2.data_ptr())   # second call, smaller input
+    fresh.synchronize()
+    free2 = torch.cuda.mem_get_info()[0]
+    assert free0 == free1 == free2, (free0, free1, free2)
+    assert amm.last_gather_kernel().startswith("gather_i8_kernel<64,")
+    assert np.array_equal(got1.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(got2.cpu().numpy().view(np.uint32), want[:200].view(np.uint32))
+    # and the existing entry point gives the same bits
+    ref = torch.empty((N, M), device="cuda")
+    amm.run_ptr(xd.data_ptr(), N, ref.data_ptr())
+    fresh.synchronize()
+    assert np.array_equal(ref.cpu().numpy().view(np.uint32), want.view(np.uint32))
+    amm.close()
+    wamm.close()
+    fresh.close()
+    warm.close()
 
 
 def test_noalloc_fp32_table(ctx):
