@@ -375,6 +375,10 @@ PIMDL_API int pimdl_amm_last_gather_kernel(const pimdl_amm* amm, char* name, siz
  * (b) a ds_read_b128 loop that keeps every CU's LDS busy.  Either pointer may be NULL. */
 PIMDL_API int pimdl_diag_bandwidth(pimdl_ctx* ctx, uint64_t bytes, float* copy_gbps,
                                    float* lds_gbps);
+/* Rates of the four legs of the host-buffer path over `bytes` bytes, GB/s: the host thread pool's copy from pageable
+ * into pinned memory and back, and the transfers between pinned memory and the device.  A measuring aid. */
+PIMDL_API int pimdl_diag_host_copy(pimdl_ctx* ctx, uint64_t bytes, float* to_pinned_gbps, float* from_pinned_gbps,
+                                   float* h2d_gbps, float* d2h_gbps);
 /* Checks on this device what the bf16-split closest-centroid search takes for granted about the
  * matrix core: runs `trials` (1..4096) chains of three v_mfma_f32_32x32x16_bf16 on random operands of
  * mixed magnitude and reports the largest |result - exact sum| in units of 2^-24 * sum|terms|.  The

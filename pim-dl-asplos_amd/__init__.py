@@ -13,7 +13,8 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libpimdl.so")
+# PIMDL_LIB_PATH: another build of the library (e.g. one compiled with other flags) instead of the in-tree one
+LIB_PATH = os.environ.get("PIMDL_LIB_PATH") or os.path.join(_HERE, "libpimdl.so")
 CSRC = os.path.join(_HERE, "csrc")
 
 LUT_I8, LUT_F32 = 0, 1
@@ -33,7 +34,7 @@ EXPORTS = ["pimdl_init", "pimdl_destroy", "pimdl_last_error", "pimdl_set_stream"
            "pimdl_diag_mfma_error", "pimdl_amm_group_create", "pimdl_amm_group_run", "pimdl_amm_group_destroy",
            "pimdl_attention", "pimdl_amm_group_fused_cols", "pimdl_amm_group_run_fused", "pimdl_amm_run_noalloc", "pimdl_amm_set_bias",
            "pimdl_amm_create_with", "pimdl_amm_set_tuning", "pimdl_amm_get_tuning", "pimdl_lutgen_mode",
-           "pimdl_diag_mfma_error_crafted", "pimdl_amm_last_gather_kernel", "pimdl_amm_run_breakdown"]
+           "pimdl_diag_mfma_error_crafted", "pimdl_amm_last_gather_kernel", "pimdl_amm_run_breakdown", "pimdl_diag_host_copy"]
 NOALLOC_SCRATCH_BYTES = 8 << 20
 
 
@@ -212,6 +213,13 @@ class Context:
         self._check(lib().pimdl_get_device_info(self._h, ctypes.byref(info)))
         return {"name": info.name.decode(), "arch": info.arch.decode(), "compute_units": info.compute_units,
                 "clock_khz": info.clock_khz, "lds_bytes_per_cu": info.lds_bytes_per_cu, "hbm_bytes": info.hbm_bytes}
+
+    def diag_host_copy(self, nbytes=100 << 20):
+        """GB/s of: pageable -> pinned and pinned -> pageable copies by the host thread pool, pinned -> device, device -> pinned."""
+        r = [ctypes.c_float() for _ in range(4)]
+        lib().pimdl_diag_host_copy.argtypes = [ctypes.c_void_p, ctypes.c_uint64] + [ctypes.POINTER(ctypes.c_float)] * 4
+        self._check(lib().pimdl_diag_host_copy(self._h, nbytes, *[ctypes.byref(x) for x in r]))
+        return dict(zip(("to_pinned_gbps", "from_pinned_gbps", "h2d_gbps", "d2h_gbps"), (x.value for x in r)))
 
     def diag_bandwidth(self, nbytes=1 << 30, copy=True, lds=True):
         c, l = ctypes.c_float(0), ctypes.c_float(0)

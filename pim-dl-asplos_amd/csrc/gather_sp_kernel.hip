@@ -18,9 +18,10 @@
 //             0..7) and 2g+1 (value bytes 8..15): each codebook is four groups of two value slots; the group
 //             that contains the token's centroid c (group c / 4) has value 1 in its first slot with position
 //             c % 4, everything else is 0.  Both codebooks' nibbles are one byte of the packed index row.
-//             The 8 value bytes of a nibble come from a 256-byte table in LDS (entry c, 16 bytes apart: 8-byte
-//             reads of such entries do not meet in a bank), the lane's whole position word (16 bits per nibble)
-//             from a second table with one 4-byte word per value of the index byte.
+//             The 8 value bytes of a nibble are the 64-bit number 1 << 16 (c / 4): one shift.  (With 17..32
+//             centroids they come from a table in LDS, entry c 16 bytes apart: 8-byte reads of such entries do
+//             not meet in a bank.)  The lane's whole position word (16 bits per nibble) comes from a second
+//             table with one 4-byte word per value of the index byte.
 //   dense B (K x columns)  lane (g, j) holds column j's 16 centroid entries of codebook g (bytes 0..15) and
 //             of codebook g + 4 (bytes 16..31): two 16-byte reads of the tiled table, whose layout is that
 //             of the dense one-hot kernel ([column tile][codebook][column][16 centroids]).
@@ -66,13 +67,24 @@ typedef int v2i __attribute__((ext_vector_type(2)));
 // SIMD, but a LUT slice is copied into LDS once for 512 tokens instead of 256 and the CU's whole LDS belongs
 // to one workgroup (slices twice as deep, half as many barriers).
 constexpr int sp_tok_item(int tm, int nw = 4) { return nw * tm * 16; }
+// workgroups per CU: two of four waves or one of eight, two waves per SIMD either way.  (Eight waves of 32 tokens
+// each, two such workgroups per CU -- four waves per SIMD on 128 registers -- were measured 17 % slower on 64-column
+// tiles: a wave then re-reads every table entry for two token groups instead of four, and 96-column tiles spill.)
+constexpr int sp_wgs_per_cu(int, int nw) { return nw == 4 ? 2 : 1; }
+// 64-token index blocks a workgroup keeps per slice: a wave of 32 tokens shares its block with its neighbour (both
+// copy the same bytes to the same place)
+constexpr int sp_ix_blocks(int tm, int nw) { return nw * tm * 16 / 64; }
 constexpr int sp_nbuf(int gs) { return gs > 16 ? 2 : 3; }
-// value table(s): 16 entries of 16 bytes, or two tables of 32; then the position words, one per index byte
-constexpr int sp_value_table_bytes(bool wide) { return wide ? 1024 : 256; }
+// value tables (17..32 centroids only: two tables of 32 entries of 16 bytes); then the position words, one per index byte
+constexpr int sp_value_table_bytes(bool wide) { return wide ? 1024 : 0; }
 constexpr int sp_table_bytes(bool wide) { return sp_value_table_bytes(wide) + 1024; }
 constexpr int sp_lds_bytes(int tn, int gs, int nw = 4, bool wide = false)
 {
     return sp_table_bytes(wide) + sp_nbuf(gs) * gs * 16 * tn * 16 + sp_nbuf(gs) * nw * 64 * 4 * (gs / 8);
+}
+constexpr int sp_lds_bytes_tm(int tn, int tm, int gs, int nw, bool wide)
+{
+    return sp_table_bytes(wide) + sp_nbuf(gs) * gs * 16 * tn * 16 + sp_nbuf(gs) * sp_ix_blocks(tm, nw) * 64 * 4 * (gs / 8);
 }
 
 template <int OFF>
@@ -102,7 +114,7 @@ __device__ __forceinline__ T* uniform_ptr(T* p)
 
 // CB_pad: codebooks of 16 centroids in the tiled table (twice the operator's for WIDE)
 template <int TN, int TM, int GS, int NW, bool WIDE>
-__global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel(
+__global__ __launch_bounds__(NW * 64, sp_wgs_per_cu(TM, NW) * NW / 4 /* waves per SIMD */) void gather_sparse_kernel(
     const uint8_t* __restrict__ idx, const int8_t* __restrict__ lut, float* __restrict__ out,
     int32_t* __restrict__ acc_out, uint32_t N, uint32_t M, uint32_t CB_pad, uint32_t idx_row_bytes,
     uint32_t n_token_tiles, uint32_t n_items, Epilogue ep, XcdMap xmap)
@@ -126,10 +138,19 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel
     constexpr uint32_t POS0 = sp_value_table_bytes(WIDE);  // position words
     constexpr uint32_t BUF0 = sp_table_bytes(WIDE);
     constexpr uint32_t IBUF0 = BUF0 + NBUF * SLICE;
-    constexpr uint32_t IBYTES = SP_WAVES * 64 * 4 * IWORDS;   // index bytes of one slice (a 64-token block per wave)
+    constexpr uint32_t IBYTES = sp_ix_blocks(TM, NW) * 64 * 4 * IWORDS;   // index bytes of one slice (64-token blocks)
     constexpr uint32_t IWAVE = 64 * 4 * IWORDS;               // ... of one wave's 64 tokens
-    constexpr int IX_OPS = IWORDS;                            // 64 lanes x 4 B = 64 tokens x 1 word
+    // index words: one operation copies one word of 64 tokens (64 lanes x 4 B) or, where a slice has a multiple of
+    // four words, four of them (64 lanes x 16 B: consecutive words of a 64-token block are consecutive 256-byte
+    // pieces in the tiled index buffer and in LDS alike); fewer instructions, the same time (measured)
+    constexpr bool IX_WIDE = IWORDS % 4 == 0;
+    constexpr int IX_OPS = IX_WIDE ? IWORDS / 4 : IWORDS;
     constexpr int DMA_OPS = DMA_PER_WAVE + IX_OPS;            // memory operations per wave and slice
+    // Up to 16 centroids: the value bytes of a nibble are 1 << 16 (c / 4) as a 64-bit number, made by one shift
+    // instead of read from a table (one LDS read per token group and K-step instead of three; measured 1 - 7 %
+    // of the kernel, most on narrow column tiles).
+    constexpr bool VALU_VALUES = !WIDE;
+    constexpr int A_OPS = VALU_VALUES ? 1 : 3;                // LDS reads per token group for the sparse operand
 
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -145,9 +166,9 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel
     // two bits per slot; low nibble in the low half of the word, high nibble in the high half).
     // WIDE: table h (h = 0, 1; 512 bytes each) has entry c at byte b = 16 h + c and zero entries elsewhere.
     static_assert(NW * 64 >= 256, "one table word per thread");
-    if (threadIdx.x < (WIDE ? 256 : 64)) {
+    if (WIDE && threadIdx.x < 256) {
         const uint32_t b = (threadIdx.x >> 2) & 31, table = threadIdx.x >> 7;
-        const uint32_t c = b & 15, w = threadIdx.x & 3, grp = c >> 2, pos = c & 3;
+        const uint32_t c = b & 15, w = threadIdx.x & 3, grp = c >> 2;
         uint32_t word;
         if (w < 2) word = (grp >> 1) == w ? (1u << (16 * (grp & 1))) : 0u;  // value bytes 0..3 / 4..7: slot 2 grp
         else word = 0;
@@ -175,7 +196,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel
         if (blk > last_block) blk = last_block;  // clamp: results of such tokens are never stored
         const uint32_t op = ep.op_col_tiles ? col_of(ix_item) / ep.op_col_tiles : 0u;
         ix_base = idx + (size_t)op * ep.op_idx_stride + (size_t)blk * idx_row_bytes * 64;
-        ix_lane_off = lane * 4;
+        ix_lane_off = lane * (IX_WIDE ? 16 : 4);
     };
     // A wave copies DMA_PER_WAVE consecutive 1 KB blocks of a slice.  All of a slice's operations share one
     // global address (the wave's part of the slice, per lane) and one LDS address; the block is chosen by the
@@ -220,12 +241,16 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel
     auto ix_begin = [&](uint32_t ibuf_off, bool fetch) {
         const uint8_t* base = uniform_ptr(fetch ? ix_base : idx);  // idx itself: any 64 tokens' words, never read
         ix_src = base + ix_lane_off;
-        ix_dst = IBUF0 + ibuf_off + wave * IWAVE;
+        ix_dst = IBUF0 + ibuf_off + (wave * (TM * 16) / 64) * IWAVE;
     };
     auto ix_op = [&](auto ic) {
         constexpr int i = decltype(ic)::value;
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)ix_src,
-                                         (__attribute__((address_space(3))) void*)(smem + ix_dst), 4, 256 * i, 0);
+        if constexpr (IX_WIDE)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)ix_src,
+                                             (__attribute__((address_space(3))) void*)(smem + ix_dst), 16, 1024 * i, 0);
+        else
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)ix_src,
+                                             (__attribute__((address_space(3))) void*)(smem + ix_dst), 4, 256 * i, 0);
     };
     auto ix_advance = [&]() {
         ix_base += IWORDS * 256;
@@ -243,7 +268,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel
     // Index word k of a token holds the nibbles of codebooks 8k .. 8k+7 of the slice; this lane's two are byte g,
     // which it reads on its own (the four lane groups read the four bytes of the same word: one bank, broadcast).
     // Kept as the two table offsets, nibble * 16.
-    const uint32_t ix_lane = IBUF0 + wave * IWAVE + (((wave * (TM * 16)) & 63) + j) * 4 + g;
+    const uint32_t ix_lane = IBUF0 + (wave * (TM * 16) / 64) * IWAVE + (((wave * (TM * 16)) & 63) + j) * 4 + g;
     auto read_ix = [&](uint32_t (&raw)[TM][IWORDS], uint32_t ibuf_off) {
         const uint32_t addr = ix_lane + ibuf_off;
         static_for<0, TM * IWORDS>([&](auto ec) {
@@ -264,6 +289,9 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel
                 if constexpr (WIDE) {  // the byte is one codebook's centroid: its entry in the first and in the second table
                     lo[t][i] = raw[t][i] << 4;
                     hi[t][i] = lo[t][i] + 512;
+                } else if constexpr (VALU_VALUES) {  // the shift that makes the value bytes: 16 bits per group of four centroids
+                    lo[t][i] = (raw[t][i] << 2) & 0x30u;
+                    hi[t][i] = (raw[t][i] >> 2) & 0x30u;
                 } else {
                     lo[t][i] = (raw[t][i] << 4) & 0xF0u;
                     hi[t][i] = raw[t][i] & 0xF0u;
@@ -410,8 +438,14 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel
 #pragma unroll
             for (int t = 0; t < TM; ++t) {
                 const uint32_t e0 = iw_lo[t][ks], e1 = iw_hi[t][ks];
-                lds_read64<0>(a_lo[ks & 1][t], e0);
-                lds_read64<0>(a_hi[ks & 1][t], e1);
+                if constexpr (VALU_VALUES) {
+                    const uint64_t v0 = 1ull << e0, v1 = 1ull << e1;
+                    a_lo[ks & 1][t] = (v2i){(int)(uint32_t)v0, (int)(uint32_t)(v0 >> 32)};
+                    a_hi[ks & 1][t] = (v2i){(int)(uint32_t)v1, (int)(uint32_t)(v1 >> 32)};
+                } else {
+                    lds_read64<0>(a_lo[ks & 1][t], e0);
+                    lds_read64<0>(a_hi[ks & 1][t], e1);
+                }
                 lds_read32<POS0>(pw[ks & 1][t], iw_pos[t][ks]);
             }
         };
@@ -429,7 +463,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gather_sparse_kernel
                 // ones this column group needs (see the issue order above and below)
                 if constexpr (c == 0) lgkm_wait<2 * (TN - 1)>();
                 else if constexpr (LAST) lgkm_wait<2 * (TN - 1 - c) + RI>();
-                else lgkm_wait<2 * TN + 3 * TM - 2>();
+                else lgkm_wait<2 * TN + A_OPS * TM - 2>();
                 if constexpr (c == 0) {
 #pragma unroll
                     for (int t = 0; t < TM; ++t)
@@ -480,15 +514,15 @@ template <int TN, int TM, int GS, int NW = 4, bool WIDE = false>
 int launch_sparse_tm(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_t* d_acc, uint32_t n,
                      const Epilogue& ep)
 {
-    constexpr int LDS = sp_lds_bytes(TN, GS, NW, WIDE);
-    static_assert((NW == 4 ? 2 : 1) * LDS <= 160 * 1024, "two workgroups of four waves, or one of eight, per CU");
+    constexpr int LDS = sp_lds_bytes_tm(TN, TM, GS, NW, WIDE);
+    static_assert(sp_wgs_per_cu(TM, NW) * LDS <= 160 * 1024, "the CU's LDS holds the workgroups that its registers hold");
     constexpr int TOK_ITEM = sp_tok_item(TM, NW);
     auto kern = gather_sparse_kernel<TN, TM, GS, NW, WIDE>;
     const uint32_t cb16 = sparse_codebooks(a.g);  // codebooks of 16 centroids in the tiled table
     if (int rc = allow_dynamic_lds(ctx, reinterpret_cast<const void*>(kern), LDS, "hipFuncSetAttribute(gather_sparse)")) return rc;
     const uint32_t n_token_tiles = (n + TOK_ITEM - 1) / TOK_ITEM;
     const uint32_t n_items = n_token_tiles * (a.g.M_pad / (16 * TN));
-    uint32_t grid = ctx->prop.multiProcessorCount * (NW == 4 ? 2 : 1);
+    uint32_t grid = ctx->prop.multiProcessorCount * sp_wgs_per_cu(TM, NW);
     if (grid > n_items) grid = n_items;
     const XcdMap xmap = choose_xcd_map(a.g.M_pad / (16 * TN), n_token_tiles, grid, (uint64_t)cb16 * 16 * a.g.M_pad,
                                        (uint64_t)n * a.g.idx_row_bytes, a.g.tune_xcd_col_split);

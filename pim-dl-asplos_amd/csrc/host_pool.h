@@ -18,10 +18,12 @@ public:
     virtual ~HostPool() {}
 };
 
-// The process-wide pool.  PIMDL_COPY_THREADS sets its width (default: 8, at most the hardware's concurrency).
+// The process-wide pool.  PIMDL_COPY_THREADS sets its width (default: 4 -- more threads were slower on the
+// measured host, where the copies share the memory system with the transfers --, at most the hardware's concurrency).
 HostPool& host_pool();
 
-// memcpy cut into cache-line aligned pieces over the pool; small copies stay on the calling thread
+// memcpy with streaming stores, cut into cache-line aligned pieces over the pool; small copies stay on the
+// calling thread
 void parallel_copy(void* dst, const void* src, size_t bytes);
 
 }  // namespace pimdl

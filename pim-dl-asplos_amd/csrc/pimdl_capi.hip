@@ -262,15 +262,32 @@ static int pipe_reserve(Ctx* ctx, HostPipe* hp, size_t in_bytes, size_t out_byte
     return PIMDL_OK;
 }
 
-// tokens per chunk: about 6 MiB of the wider staged side, a multiple of 512 tokens (whole items of every gather)
-static uint32_t pipe_chunk_tokens(uint32_t n, size_t row_bytes)
+// Chunk boundaries (first token of each chunk, then n).  Chunks hold about 12 MiB of the wider staged side, in
+// multiples of 256 tokens (whole items of the gathers); the first two and the last two are a quarter and a half of
+// that, so that the device starts early and little is left to come back and be copied out after the last kernel.
+static std::vector<uint32_t> pipe_chunks(uint32_t n, size_t row_bytes)
 {
     const char* e = getenv("PIMDL_HOST_CHUNK_TOKENS");
-    uint64_t t = e ? strtoull(e, nullptr, 10) : 0;
-    if (!t) t = (6u << 20) / (row_bytes ? row_bytes : 1);
-    t = t / 512 * 512;
-    if (t < 512) t = 512;
-    return t >= n ? n : (uint32_t)t;
+    const uint64_t forced = e ? strtoull(e, nullptr, 10) : 0;
+    uint64_t base = forced ? forced : (12u << 20) / (row_bytes ? row_bytes : 1);
+    base = base / 256 * 256;
+    if (base < 256) base = 256;
+    std::vector<uint32_t> b;
+    const bool ramp = !forced && base >= 1024 && n >= 4 * base;
+    const uint32_t head[2] = {(uint32_t)base / 4, (uint32_t)base / 2};
+    uint32_t at = 0;
+    b.push_back(0);
+    if (ramp)
+        for (uint32_t h : head) b.push_back(at += h);
+    const uint32_t tail = ramp ? head[0] + head[1] : 0;
+    while (n - at > base + tail) b.push_back(at += (uint32_t)base);
+    if (ramp) {
+        const uint32_t rest = n - at - tail;  // 1 .. base tokens
+        if (rest) b.push_back(at += rest);
+        b.push_back(at += head[1]);
+    }
+    b.push_back(n);
+    return b;
 }
 
 // One AMM with at least one of in / out in host memory.  `run_chunk(d_in, d_out, tokens)` queues the kernels of
@@ -290,8 +307,15 @@ static int run_piped(Ctx* ctx, uint32_t K, uint32_t M, const float* in, bool in_
     constexpr int SLOTS = HostPipe::SLOTS, LAG = SLOTS - 1;
     const size_t in_row = (size_t)K * sizeof(float), out_row = (size_t)M * sizeof(float);
     const size_t wide = (in_host ? in_row : 0) > (out_host ? out_row : 0) ? in_row : out_row;
-    const uint32_t chunk = pipe_chunk_tokens(n, wide);
-    const uint32_t nchunks = (n + chunk - 1) / chunk;
+    std::vector<uint32_t> first;  // chunk c holds tokens first[c] .. first[c + 1] - 1
+    try {
+        first = pipe_chunks(n, wide);
+    } catch (...) {
+        return set_error(ctx, PIMDL_ERR_NOMEM, "host staging: out of host memory");
+    }
+    const uint32_t nchunks = (uint32_t)first.size() - 1;
+    uint32_t chunk = 0;  // the largest
+    for (uint32_t c = 0; c < nchunks; ++c) chunk = std::max(chunk, first[c + 1] - first[c]);
     if ((rc = pipe_reserve(ctx, hp, in_host ? chunk * in_row : 0, out_host ? chunk * out_row : 0))) return rc;
 
     auto fail = [&](int code) {  // nothing may stay in flight towards buffers the caller owns
@@ -300,13 +324,13 @@ static int run_piped(Ctx* ctx, uint32_t K, uint32_t M, const float* in, bool in_
         (void)hipStreamSynchronize(hp->s_out);
         return code;
     };
-    auto tokens_of = [&](uint32_t c) { return c + 1 == nchunks ? n - c * chunk : chunk; };
+    auto tokens_of = [&](uint32_t c) { return first[c + 1] - first[c]; };
     for (uint32_t c = 0; c < nchunks + (out_host ? LAG : 0); ++c) {
         if (c < nchunks) {
             const int s = c % SLOTS;
             const uint32_t tok = tokens_of(c);
-            const float* d_in = in + (size_t)c * chunk * K;
-            float* d_out = out + (size_t)c * chunk * M;
+            const float* d_in = in + (size_t)first[c] * K;
+            float* d_out = out + (size_t)first[c] * M;
             if (in_host) {
                 // the slot's pinned buffer is free once its last transfer has left it
                 if (hp->used_in[s] && (rc = hip_check(ctx, hipEventSynchronize(hp->ev_in[s]), "hipEventSynchronize(staging in)"))) return fail(rc);
@@ -338,7 +362,7 @@ static int run_piped(Ctx* ctx, uint32_t K, uint32_t M, const float* in, bool in_
             const uint32_t r = c - LAG;
             const int s = r % SLOTS;
             if ((rc = hip_check(ctx, hipEventSynchronize(hp->ev_out[s]), "hipEventSynchronize(staging out)"))) return fail(rc);
-            parallel_copy(out + (size_t)r * chunk * M, hp->pin_out[s], tokens_of(r) * out_row);
+            parallel_copy(out + (size_t)first[r] * M, hp->pin_out[s], tokens_of(r) * out_row);
         }
     }
     return PIMDL_OK;
@@ -1308,6 +1332,46 @@ int pimdl_diag_bandwidth(pimdl_ctx* ctx, uint64_t bytes, float* copy_gbps, float
     int rc = activate(ctx);
     if (rc) return rc;
     return launch_diag(ctx, bytes, copy_gbps, lds_gbps);
+}
+
+int pimdl_diag_host_copy(pimdl_ctx* ctx, uint64_t bytes, float* to_pinned_gbps, float* from_pinned_gbps, float* h2d_gbps,
+                         float* d2h_gbps)
+{
+    if (!ctx) return PIMDL_ERR_INVALID;
+    if (!bytes || !to_pinned_gbps || !from_pinned_gbps || !h2d_gbps || !d2h_gbps)
+        return set_error(ctx, PIMDL_ERR_INVALID, "pimdl_diag_host_copy: bad arguments");
+    int rc = activate(ctx);
+    if (rc) return rc;
+    void *pinned = nullptr, *dev = nullptr;
+    char* pageable = static_cast<char*>(malloc(bytes));
+    if (!pageable) return set_error(ctx, PIMDL_ERR_NOMEM, "pimdl_diag_host_copy: out of host memory");
+    memset(pageable, 1, bytes);
+    rc = hip_check(ctx, hipHostMalloc(&pinned, bytes, hipHostMallocDefault), "hipHostMalloc(diag)");
+    if (!rc) rc = hip_check(ctx, hipMalloc(&dev, bytes), "hipMalloc(diag)");
+    auto now = [] { return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count(); };
+    constexpr int REPS = 5;
+    auto rate = [&](auto fn, float* out) {
+        fn();
+        const double t0 = now();
+        for (int i = 0; i < REPS && !rc; ++i) fn();
+        *out = (float)((double)bytes * REPS / (now() - t0) / 1e9);
+    };
+    if (!rc) {
+        rate([&] { parallel_copy(pinned, pageable, bytes); }, to_pinned_gbps);
+        rate([&] { parallel_copy(pageable, pinned, bytes); }, from_pinned_gbps);
+        rate([&] {
+            rc = hip_check(ctx, hipMemcpyAsync(dev, pinned, bytes, hipMemcpyHostToDevice, ctx->stream), "H2D diag");
+            if (!rc) rc = hip_check(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+        }, h2d_gbps);
+        rate([&] {
+            rc = hip_check(ctx, hipMemcpyAsync(pinned, dev, bytes, hipMemcpyDeviceToHost, ctx->stream), "D2H diag");
+            if (!rc) rc = hip_check(ctx, hipStreamSynchronize(ctx->stream), "hipStreamSynchronize");
+        }, d2h_gbps);
+    }
+    if (pinned) (void)hipHostFree(pinned);
+    (void)hipFree(dev);
+    free(pageable);
+    return rc;
 }
 
 int pimdl_diag_mfma_error(pimdl_ctx* ctx, uint32_t trials, float* max_err_u)
