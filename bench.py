@@ -34,6 +34,10 @@ MEASURED_GATHER_TRAFFIC = {
     ("gather_sparse_kernel<3, 4, 64, 8, false>", 8192, 3072, 768): {"fetch_kib": 15644.5, "write_kib": 25039.7},
 }
 FETCH_SCALE, WRITE_SCALE = 2.0, 1.0
+# Busy fractions of the same kernels from a rocprofv3 --pmc run of this script (summary:
+# profiles/bench_ffn_pair_lds_mfma_counters.txt): matrix core (SQ_VALU_MFMA_BUSY_CYCLES / SQ_BUSY_CU_CYCLES), LDS
+# (SQ_LDS_IDX_ACTIVE / ...), LDS bank-conflict cycles over LDS-active cycles.  Reported only for the kernel they belong to.
+MEASURED_GATHER_COUNTERS = {}
 CLOCK_SETTLE_S = 0.08                      # untimed pre-heat: the engine clock needs ~20 ms of this load to ramp up
 
 
@@ -190,6 +194,23 @@ def cpu_baseline(shapes, N, warmup=10, rounds=20, budget_s=25.0):
                       f"flags (-O3 -fopenmp, no -march), {threads} OpenMP threads, {dt * 1e3:.1f} ms per round"}
 
 
+def check_pair(amms, shapes, x1, x2, h, y, N, sample=64):
+    """Bit-compares `sample` rows of both outputs of the timed step with the oracle's amm_cpu on the same inputs
+    (indices, int32 sums and the fp32 epilogue all enter the compared bits).  Raises on a mismatch."""
+    import oracle
+    rows = np.sort(np.random.default_rng(5).choice(N, size=sample, replace=False))
+    rows[0], rows[-1] = 0, N - 1
+    for amm, (K, v, C, M), x, out in zip(amms, shapes, (x1, x2), (h, y)):
+        xs = x[rows].cpu().numpy()
+        got = out[rows].cpu().numpy()
+        want, _, _ = oracle.amm_cpu(xs, amm.h_centroids, amm.h_lut, amm.h_bias, v, float(amm.h_scales[0]), 0.0,
+                                    threads=min(16, oracle.max_threads()))
+        if not np.array_equal(got.view(np.uint32), want.view(np.uint32)):
+            bad = int((got.view(np.uint32) != want.view(np.uint32)).sum())
+            raise SystemExit(f"bench.py: the timed {K}->{M} launch differs from the oracle in {bad} of {want.size} sampled outputs")
+    return True
+
+
 def settled_profile(amm, x, N, y, iters):
     """pimdl_amm_profile after enough warm-up launches (about 30 ms of them) for the engine clock to have ramped
     up again: preparing an operator on the host leaves the GPU idle for a second, and the clock drops meanwhile."""
@@ -290,7 +311,9 @@ def main():
     amms = []
     for (K, vv, CC, M) in shapes:
         cent, lut, scales, bias = synth_amm(rng, K, vv, CC, M, pimdl, ctx)
-        amms.append(ctx.amm(cent, lut, scales, bias, max_n=N))
+        amm = ctx.amm(cent, lut, scales, bias, max_n=N)
+        amm.h_centroids, amm.h_lut, amm.h_scales, amm.h_bias = cent, lut, np.atleast_1d(scales), bias   # for check_pair
+        amms.append(amm)
 
     gen = torch.Generator(device="cuda").manual_seed(0)
     x1 = torch.randn((N, 768), device="cuda", generator=gen, dtype=torch.float32)
@@ -331,6 +354,10 @@ def main():
     ev_ms = e0.elapsed_time(e1) / args.steps
     ms_per_step = wall_ms
 
+    # The outputs the timed steps left behind, against the oracle on a 64-row sample (rows are independent): the
+    # exact launches that were timed, not a separate test run.
+    checked = check_pair(amms, shapes, x1, x2, h, y, N)
+
     # per-kernel device times: HIP events on the launch stream, each kernel launched on its own (pimdl_amm_profile)
     prof = [amms[0].profile(x1.data_ptr(), N, h.data_ptr(), warmup=200, iters=max(50, args.steps)),
             amms[1].profile(x2.data_ptr(), N, y.data_ptr(), warmup=200, iters=max(50, args.steps))]
@@ -369,6 +396,10 @@ def main():
     roofline = {
         "kernel": f"{dom['gather_kernel']} ({dom['name']}: K={K} M={M})",
         "bound": "lds",
+        "kind": "algorithmic",   # N*CB*M gathered bytes per launch over the LDS read peak: the roofline the metric is
+                                 # worded in.  The kernel gathers through one-hot products on the sparse matrix
+                                 # instruction and does not move those bytes through LDS; the units it does occupy are
+                                 # under "matrix_core" and "lds_counters" (utilisation, not rooflines).
         "achieved": dom["gather_lds_gbps"], "peak": LDS_PEAK_GBPS, "unit": "GB/s", "frac": dom["gather_lds_frac"],
         "algorithmic_bytes_per_launch": ab["gather_lds"],
         "avg_launch_ms": dom["gather_ms"],
@@ -388,6 +419,12 @@ def main():
                         "dense_int8_peak_tops": MFMA_I8_PEAK_TOPS},
         "north_star_target_frac": 0.5,
     }
+    lc = MEASURED_GATHER_COUNTERS.get((dom["gather_kernel"], N, K, M))
+    roofline["lds_counters"] = dict(lc, source="rocprofv3 --pmc of this script for this kernel and batch; "
+                                    "profiles/bench_ffn_pair_lds_mfma_counters.txt") if lc else None
+    # the step as a whole on the same roofline: both gathers' algorithmic bytes over the whole step (searches included)
+    step_lds = sum(algorithmic_bytes(N, K_, v, C, M_)["gather_lds"] for (K_, _, _, M_) in shapes)
+    roofline["step_frac"] = step_lds / (ms_per_step * 1e-3) / 1e9 / LDS_PEAK_GBPS
 
     total_eff_ops = sum(algorithmic_bytes(N, K_, v, C, M_)["eff_ops"] for (K_, _, _, M_) in shapes)
     result = {
@@ -412,23 +449,44 @@ def main():
     # A labelled secondary figure; `value` above is the HBM-resident rate.
     xh = np.random.default_rng(1).standard_normal((N, 768)).astype(np.float32)
     hh, yh = np.empty((N, 3072), np.float32), np.empty((N, 768), np.float32)
-    for it in range(4):
-        if it == 1:
-            t0 = time.perf_counter()
+    host_steps = []
+    for it in range(8):
+        t0 = time.perf_counter()
         amms[0].run_ptr(xh.ctypes.data, N, hh.ctypes.data)
         amms[1].run_ptr(hh.ctypes.data, N, yh.ctypes.data)
-    host_ms = (time.perf_counter() - t0) * 1e3 / 3
-    result["host_buffers"] = {"ms_per_step": host_ms, "tokens_per_s": N / (host_ms * 1e-3),
-                              "note": "pageable host memory in and out of both AMMs (PCIe copies included), 3 steps"}
+        host_steps.append((time.perf_counter() - t0) * 1e3)
+    host_ms = float(np.mean(host_steps[3:]))   # the first steps fault the fresh host buffers in and size the staging ring
+    legs = ctx.diag_host_copy(100 << 20)
+    link_floor_ms = sum(4.0 * N * max(K_, M_) for (K_, _, _, M_) in shapes) / (min(legs["h2d_gbps"], legs["d2h_gbps"]) * 1e9) * 1e3
+    host_buffers = {"ms_per_step": host_ms, "tokens_per_s": N / (host_ms * 1e-3), "steps_ms": [round(t, 2) for t in host_steps],
+                    "legs_gbps": {k: round(val, 1) for k, val in legs.items()},
+                    "link_floor_ms": link_floor_ms,
+                    "note": "pageable host memory in and out of both AMMs (what the reference's amm_host signature hands "
+                            "over), mean of the last 5 of 8 steps: chunks of tokens through pinned staging buffers, copies by the host thread "
+                            "pool, transfers and kernels overlapped on three streams.  link_floor_ms: the wider side of "
+                            "each AMM (100 MB) over the measured pinned-memory link rate, both directions overlapped"}
+    # The large objects first, the small ones last (a reader that keeps only the end of the line keeps those).
+    if not args.no_sweep:
+        result["vit_base_sweep"] = vit_sweep(pimdl, ctx)
+        result["per_codebook_scale"] = per_codebook_scale(pimdl, ctx, rng, N, shapes)
+    result["host_buffers"] = host_buffers
     if not args.no_model:
-        result["bert_base_forward"] = model_forward(pimdl, ctx)
         if not args.no_large_layer:
             result["bert_large_layer"] = bert_large_layer(pimdl, ctx)
-    if not args.no_sweep:
-        result["per_codebook_scale"] = per_codebook_scale(pimdl, ctx, rng, N, shapes)
-        result["vit_base_sweep"] = vit_sweep(pimdl, ctx)
+        result["bert_base_forward"] = model_forward(pimdl, ctx)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(shapes, N)
+    result["checked"] = checked
+    result["summary"] = {
+        "tokens_per_s": result["value"], "ms_per_step": ms_per_step, "checked_against_oracle": checked,
+        "roofline_frac": roofline["frac"], "roofline_step_frac": roofline["step_frac"],
+        "gather_us": [round(p["gather_ms"] * 1e3, 1) for p in per_amm], "search_us": [round(p["ccs_ms"] * 1e3, 1) for p in per_amm],
+        "host_buffers_ms": round(host_ms, 2),
+        "bert_base_forward_ms": round(result["bert_base_forward"]["ms_per_forward_graph"], 3) if "bert_base_forward" in result else None,
+        "bert_large_layer_ms": round(result["bert_large_layer"]["ms_per_layer"], 3) if "bert_large_layer" in result else None,
+        "per_codebook_scale_ms": round(result["per_codebook_scale"]["ms_per_step"], 3) if "per_codebook_scale" in result else None,
+        "cpu_tokens_per_s": round(result["cpu_baseline"]["value"]) if "cpu_baseline" in result else None,
+    }
     for a in amms:
         a.close()
     ctx.close()
