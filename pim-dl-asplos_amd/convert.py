@@ -72,7 +72,12 @@ def linear_shape(op_name, features):
 def convert(tensors, ctx, pimdl, features=768, ncentroids=16, vec_len=2, nsharecodebook=1, lut_dtype="int8",
             ordered_sum=False):
     if nsharecodebook != 1:
-        raise ValueError("nsharecodebook != 1 is not supported (the inference engine has one codebook per sub-vector)")
+        # The reference divides the codebook count by it (pim_weight_converter.py:82, LUTLinear_t.py:26) and then views
+        # the [in][out] weight and the activations as [ncodebooks][vec_len][...] (pim_weight_converter.py:86,
+        # LUTLinear_t.py:68-69), which only has the right number of elements for 1: its own code raises for any other
+        # value, and its inference engine has one codebook per sub-vector (index_calc_host.cpp:22).
+        raise ValueError("nsharecodebook != 1 is not supported: the reference's own converter and LUTLinear_t.forward fail "
+                         "on it (a [in][out] weight cannot be viewed as [in/vec_len/nsharecodebook][vec_len][out])")
     layers = split_layers(tensors)
     out = {}
     for _li, lt in sorted(layers.items()):
