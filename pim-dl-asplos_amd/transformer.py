@@ -292,6 +292,13 @@ class Transformer:
         self.layers = [TransformerLayer(ctx, pimdl, w, params, fused_qkv, self.side, fused_gelu) for w in layers]
         self.params = params
 
+    @classmethod
+    def from_layers(cls, layers, params):
+        """A model over TransformerLayer objects that already exist (they stay the caller's to close)."""
+        self = cls.__new__(cls)
+        self.side, self.layers, self.params = None, list(layers), params
+        return self
+
     def close(self):
         for layer in self.layers:
             layer.close()
