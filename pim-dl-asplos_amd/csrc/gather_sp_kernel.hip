@@ -276,28 +276,13 @@ __global__ __launch_bounds__(NW * 64, sp_wgs_per_cu(TM, NW) * NW / 4 /* waves pe
             lds_read_u8<(i * 64 + t * 16) * 4>(raw[t][i], addr);
         });
     };
-    auto unpack_ix = [&](uint32_t (&lo)[TM][IWORDS], uint32_t (&hi)[TM][IWORDS], uint32_t (&pa)[TM][IWORDS], uint32_t (&raw)[TM][IWORDS]) {
+    // the index bytes requested by read_ix have landed (the registers pass through the wait)
+    auto wait_ix = [&](uint32_t (&raw)[TM][IWORDS]) {
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
         for (int t = 0; t < TM; ++t)
 #pragma unroll
             for (int i = 0; i < IWORDS; ++i) asm volatile("" : "+v"(raw[t][i]));
-#pragma unroll
-        for (int t = 0; t < TM; ++t)
-#pragma unroll
-            for (int i = 0; i < IWORDS; ++i) {
-                if constexpr (WIDE) {  // the byte is one codebook's centroid: its entry in the first and in the second table
-                    lo[t][i] = raw[t][i] << 4;
-                    hi[t][i] = lo[t][i] + 512;
-                } else if constexpr (VALU_VALUES) {  // the shift that makes the value bytes: 16 bits per group of four centroids
-                    lo[t][i] = (raw[t][i] << 2) & 0x30u;
-                    hi[t][i] = (raw[t][i] >> 2) & 0x30u;
-                } else {
-                    lo[t][i] = (raw[t][i] << 4) & 0xF0u;
-                    hi[t][i] = raw[t][i] & 0xF0u;
-                }
-                pa[t][i] = raw[t][i] << 2;  // its position word
-            }
     };
 
     v4i acc[TM][TN];
@@ -393,9 +378,9 @@ __global__ __launch_bounds__(NW * 64, sp_wgs_per_cu(TM, NW) * NW / 4 /* waves pe
     });
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();  // also: the table is complete
-    uint32_t iw_lo[TM][IWORDS], iw_hi[TM][IWORDS], iw_pos[TM][IWORDS], iw_raw[TM][IWORDS];
+    uint32_t iw_raw[TM][IWORDS];
     read_ix(iw_raw, 0);
-    unpack_ix(iw_lo, iw_hi, iw_pos, iw_raw);
+    wait_ix(iw_raw);
 
     uint32_t item0 = blockIdx.x;
     const uint32_t b_lane = BUF0 + (g * WN + j) * 16;  // this lane's 16 bytes of codebook g, column position j
@@ -433,20 +418,27 @@ __global__ __launch_bounds__(NW * 64, sp_wgs_per_cu(TM, NW) * NW / 4 /* waves pe
             lds_read<((8 * ks) * WN + c * 16) * 16>(b_lo[c], bbase);
             lds_read<((8 * ks + 4) * WN + c * 16) * 16>(b_hi[c], bbase);
         };
+        // The sparse operand of K-step ks from the index bytes: what a byte turns into is worked out here, between the
+        // matrix instructions of the K-step before (a few vector operations per token group in their shadow), not for
+        // the whole slice at its boundary, where a wave would spend them alone.
         auto issue_a = [&](auto ksc) {
             constexpr int ks = decltype(ksc)::value;
 #pragma unroll
             for (int t = 0; t < TM; ++t) {
-                const uint32_t e0 = iw_lo[t][ks], e1 = iw_hi[t][ks];
+                const uint32_t raw = iw_raw[t][ks];
+                const uint32_t pa = raw << 2;  // its position word
                 if constexpr (VALU_VALUES) {
-                    const uint64_t v0 = 1ull << e0, v1 = 1ull << e1;
+                    // the shift that makes the value bytes: 16 bits per group of four centroids
+                    const uint64_t v0 = 1ull << (pa & 0x30u), v1 = 1ull << ((raw >> 2) & 0x30u);
                     a_lo[ks & 1][t] = (v2i){(int)(uint32_t)v0, (int)(uint32_t)(v0 >> 32)};
                     a_hi[ks & 1][t] = (v2i){(int)(uint32_t)v1, (int)(uint32_t)(v1 >> 32)};
                 } else {
+                    // (17..32 centroids) the byte is one codebook's centroid: its entry in the first and in the second table
+                    const uint32_t e0 = raw << 4;
                     lds_read64<0>(a_lo[ks & 1][t], e0);
-                    lds_read64<0>(a_hi[ks & 1][t], e1);
+                    lds_read64<512>(a_hi[ks & 1][t], e0);
                 }
-                lds_read32<POS0>(pw[ks & 1][t], iw_pos[t][ks]);
+                lds_read32<POS0>(pw[ks & 1][t], pa);
             }
         };
         // slice prologue: sparse operand first, then the dense operand of every column group, in this order
@@ -499,7 +491,7 @@ __global__ __launch_bounds__(NW * 64, sp_wgs_per_cu(TM, NW) * NW / 4 /* waves pe
             lut_advance();
             if (fetch_ix) ix_advance();
         }
-        unpack_ix(iw_lo, iw_hi, iw_pos, iw_raw);
+        wait_ix(iw_raw);
 
         copy_off = cur_off;
         cur_off = cur_off + SLICE == NBUF * SLICE ? 0 : cur_off + SLICE;
