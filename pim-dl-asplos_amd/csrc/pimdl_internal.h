@@ -33,8 +33,9 @@ struct AmmGeom {
     uint32_t lut_chunked;   // fp32 table of 32 centroids: [column block][codebook][8-byte chunk][row][2 floats]
     // gather kernel
     uint32_t gather_kind;   // 0: byte-adder rows kernel, 1: one-hot matrix-core kernel (int8, C <= 16),
-                            // 2: one-hot on the sparse matrix instruction (int8, 9 <= C <= 16; table laid out
-                            //    as for 1, with the columns of a tile permuted by sparse_tile_column)
+                            // 2: one-hot on the sparse matrix instruction (int8, C <= 32: a codebook of 17..32
+                            //    centroids is two of 16 side by side; table laid out as for 1, with the columns
+                            //    of a tile permuted by sparse_tile_column)
     uint32_t q;             // 16-byte chunks per LUT row in LDS
     uint32_t col_block;     // columns per workgroup (int8: 16*q, fp32: 4*q)
     uint32_t row_pitch;     // bytes between LUT rows in LDS (16*q + 16: bank-conflict-free b128 gathers)
