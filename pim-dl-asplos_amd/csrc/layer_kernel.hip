@@ -54,7 +54,8 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const float* __restrict
 }
 
 // The same for rows of up to 64 * 4 * KV floats with d % 4 == 0 and 16-byte aligned buffers: the row
-// is read once with float4 loads and stays in registers for the three passes.
+// is read once with float4 loads and stays in registers for the three passes.  Weight, bias and residual are
+// requested together with the row, ahead of the two reductions, so that the wave waits for memory once.
 template <int KV>
 __global__ __launch_bounds__(256) void layer_norm_vec_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                             const float* __restrict__ b,
@@ -66,13 +67,25 @@ __global__ __launch_bounds__(256) void layer_norm_vec_kernel(const float* __rest
     if (row >= n) return;
     const uint32_t d4 = d / 4;
     const float4* xr = reinterpret_cast<const float4*>(x + (size_t)row * d);
-    float4 xv[KV];
-    double s = 0.0;
+    float4 xv[KV], wv[KV], bv[KV], rv[KV];
+    const float4* r = residual ? reinterpret_cast<const float4*>(residual + (size_t)row * d) : nullptr;
+    const float4* w4 = reinterpret_cast<const float4*>(w);
+    const float4* b4 = reinterpret_cast<const float4*>(b);
 #pragma unroll
     for (int k = 0; k < KV; ++k) {
         const uint32_t i = lane + 64 * k;
         if (i < d4) {
             xv[k] = xr[i];
+            wv[k] = w4[i];
+            bv[k] = b4[i];
+            if (r) rv[k] = r[i];
+        }
+    }
+    double s = 0.0;
+#pragma unroll
+    for (int k = 0; k < KV; ++k) {
+        const uint32_t i = lane + 64 * k;
+        if (i < d4) {
             s += (double)xv[k].x;
             s += (double)xv[k].y;
             s += (double)xv[k].z;
@@ -97,25 +110,20 @@ __global__ __launch_bounds__(256) void layer_norm_vec_kernel(const float* __rest
     const float variance = (float)(wave_sum(s2) / (double)d);
     const float scale = 1.0f / sqrtf(__fadd_rn(variance, eps));
     float4* o = reinterpret_cast<float4*>(out + (size_t)row * d);
-    const float4* r = residual ? reinterpret_cast<const float4*>(residual + (size_t)row * d) : nullptr;
-    const float4* w4 = reinterpret_cast<const float4*>(w);
-    const float4* b4 = reinterpret_cast<const float4*>(b);
 #pragma unroll
     for (int k = 0; k < KV; ++k) {
         const uint32_t i = lane + 64 * k;
         if (i < d4) {
-            const float4 wv = w4[i], bv = b4[i];
             float4 y;
-            y.x = __fadd_rn(__fmul_rn(__fmul_rn(xv[k].x, scale), wv.x), bv.x);
-            y.y = __fadd_rn(__fmul_rn(__fmul_rn(xv[k].y, scale), wv.y), bv.y);
-            y.z = __fadd_rn(__fmul_rn(__fmul_rn(xv[k].z, scale), wv.z), bv.z);
-            y.w = __fadd_rn(__fmul_rn(__fmul_rn(xv[k].w, scale), wv.w), bv.w);
+            y.x = __fadd_rn(__fmul_rn(__fmul_rn(xv[k].x, scale), wv[k].x), bv[k].x);
+            y.y = __fadd_rn(__fmul_rn(__fmul_rn(xv[k].y, scale), wv[k].y), bv[k].y);
+            y.z = __fadd_rn(__fmul_rn(__fmul_rn(xv[k].z, scale), wv[k].z), bv[k].z);
+            y.w = __fadd_rn(__fmul_rn(__fmul_rn(xv[k].w, scale), wv[k].w), bv[k].w);
             if (r) {
-                const float4 rv = r[i];
-                y.x = __fadd_rn(rv.x, y.x);
-                y.y = __fadd_rn(rv.y, y.y);
-                y.z = __fadd_rn(rv.z, y.z);
-                y.w = __fadd_rn(rv.w, y.w);
+                y.x = __fadd_rn(rv[k].x, y.x);
+                y.y = __fadd_rn(rv[k].y, y.y);
+                y.z = __fadd_rn(rv[k].z, y.z);
+                y.w = __fadd_rn(rv[k].w, y.w);
             }
             o[i] = y;
         }
