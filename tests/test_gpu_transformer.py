@@ -40,7 +40,7 @@ def amm_oracle(w, x):
     return oracle.dequant(acc, w["bias"], CB, w["scale"], w.get("lut_bias", 0.0), 1, threads=8)
 
 
-@pytest.mark.parametrize("n,d", [(1, 8), (37, 768), (256, 1024), (5, 100), (3, 4097)])
+@pytest.mark.parametrize("n,d", [(1, 8), (37, 768), (256, 1024), (5, 100), (3, 4097), (9, 2048), (6, 1540)])
 def test_layer_norm_matches_the_reference_statement(ctx, n, d):
     rng = np.random.default_rng(n * 1000 + d)
     x = (rng.standard_normal((n, d)) * 3 + 0.5).astype(np.float32)
