@@ -100,7 +100,7 @@ private:
 
 int pool_width()
 {
-    int w = 4;
+    int w = 8;
     if (const char* e = getenv("PIMDL_COPY_THREADS")) w = atoi(e);
     const int hw = (int)std::thread::hardware_concurrency();
     if (hw > 0 && w > hw) w = hw;
@@ -178,7 +178,7 @@ static int copy_mode()
 {
     static const int mode = [] {
         const char* e = getenv("PIMDL_COPY_MODE");
-        int m = e ? atoi(e) : 0;
+        int m = e ? atoi(e) : 1;
         if (m == 2 && !__builtin_cpu_supports("avx2")) m = 1;
         return m;
     }();
