@@ -152,8 +152,10 @@ typedef struct pimdl_amm_tuning {
     uint32_t token_item;     /* tokens per work item of the matrix-core gathers: 128 or 256; the sparse kernel
                                 also 512 (one workgroup of eight waves per CU instead of two of four) */
     uint32_t cb_per_slice;   /* codebooks staged in LDS at a time by the matrix-core gathers: 16 or 32
-                                (32 needs col_block <= 64, or 512-token items); 64 with 512-token items and
-                                col_block 48, num_codebook padded to a multiple of 64 */
+                                (32 needs col_block <= 64, or 512-token items); 64 with col_block 48 and
+                                num_codebook padded to a multiple of 64, for 512-token items or for 256-token
+                                items (eight waves either way; with 256 tokens the two waves of a SIMD share
+                                their tokens and split the slice's codebooks) */
     uint32_t xcd_col_split;  /* how the 8 XCDs (each with its own L2) share the work items of the matrix-core
                                 gathers: 1, 2, 4 or 8 of them along the column tiles, the rest along the token
                                 tiles; PIMDL_XCD_PLAIN = no dealing.  A split that does not divide a launch's

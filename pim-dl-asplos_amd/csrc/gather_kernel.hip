@@ -1185,7 +1185,9 @@ bool apply_runtime_tuning(AmmGeom* g, const pimdl_amm_tuning& t, std::string* wh
     if (t.cb_per_slice) {
         const uint32_t entries = g->C_tile == 8 ? g->CB_pad / 2 : g->C_tile == 32 ? 2 * g->CB_pad : g->CB_pad;  // table entries of 16 slots
         const bool has32 = eight_waves || (g->gather_kind == 2 ? g->q <= 4 : (g->q == 3 || (g->q == 4 && g->C_tile != 8)));
-        const bool has64 = eight_waves && g->q == 3;
+        // 64-codebook slices: eight waves, either 512-token items or 256-token items whose two waves of a SIMD
+        // split the slice between them
+        const bool has64 = g->q == 3 && (eight_waves || (t.token_item == 256 && g->gather_kind == 2 && g->C_tile != 32));
         if (!matrix_core || (t.cb_per_slice == 16 && eight_waves && g->q == 3) ||
             (t.cb_per_slice != 16 && !(t.cb_per_slice == 32 && has32 && entries % 32 == 0) &&
                              !(t.cb_per_slice == 64 && has64 && entries % 64 == 0))) {

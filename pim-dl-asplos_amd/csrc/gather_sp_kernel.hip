@@ -82,9 +82,10 @@ constexpr int sp_lds_bytes(int tn, int gs, int nw = 4, bool wide = false)
 {
     return sp_table_bytes(wide) + sp_nbuf(gs) * gs * 16 * tn * 16 + sp_nbuf(gs) * nw * 64 * 4 * (gs / 8);
 }
-constexpr int sp_lds_bytes_tm(int tn, int tm, int gs, int nw, bool wide)
+// ks: waves that share a token block and split the codebooks of a slice between them (1 or 2)
+constexpr int sp_lds_bytes_tm(int tn, int tm, int gs, int nw, bool wide, int ks = 1)
 {
-    return sp_table_bytes(wide) + sp_nbuf(gs) * gs * 16 * tn * 16 + sp_nbuf(gs) * sp_ix_blocks(tm, nw) * 64 * 4 * (gs / 8);
+    return sp_table_bytes(wide) + sp_nbuf(gs) * gs * 16 * tn * 16 + sp_nbuf(gs) * sp_ix_blocks(tm, nw / ks) * 64 * 4 * (gs / 8);
 }
 
 template <int OFF>
@@ -113,20 +114,26 @@ __device__ __forceinline__ T* uniform_ptr(T* p)
 }
 
 // CB_pad: codebooks of 16 centroids in the tiled table (twice the operator's for WIDE)
-template <int TN, int TM, int GS, int NW, bool WIDE>
+// KS = 2 (eight waves): waves w and w + 4 hold the same 64 tokens and take one half of every slice's codebooks each;
+// the halves are added through LDS before the epilogue.  An item is then 256 tokens: a launch too small to give
+// every CU a 512-token item still fills the chip with TM = 4 tiles and copies a slice once per 256 tokens.
+template <int TN, int TM, int GS, int NW, bool WIDE, int KS = 1>
 __global__ __launch_bounds__(NW * 64, sp_wgs_per_cu(TM, NW) * NW / 4 /* waves per SIMD */) void gather_sparse_kernel(
     const uint8_t* __restrict__ idx, const int8_t* __restrict__ lut, float* __restrict__ out,
     int32_t* __restrict__ acc_out, uint32_t N, uint32_t M, uint32_t CB_pad, uint32_t idx_row_bytes,
     uint32_t n_token_tiles, uint32_t n_items, Epilogue ep, XcdMap xmap)
 {
     constexpr int SP_WAVES = NW;
-    constexpr int TOK_ITEM = sp_tok_item(TM, NW);
+    constexpr int NWT = NW / KS;                   // waves with tokens of their own
+    static_assert(KS == 1 || (KS == 2 && NW == 8), "the codebook split is between the two waves of a SIMD");
+    constexpr int TOK_ITEM = sp_tok_item(TM, NWT);
     static_assert(TM == 4 || TM == 2, "a wave owns a whole or half a 64-token index block");
     constexpr int WN = 16 * TN;                    // columns per item
     constexpr int G = GS;                          // codebooks per slice
     constexpr int SLICE = G * WN * 16;             // bytes of one codebook slice
-    constexpr int KSTEPS = G / 8;                  // one instruction covers 8 codebooks
-    constexpr int IWORDS = G / 8;                  // 32-bit index words per token and slice (8 nibbles each)
+    constexpr int KSTEPS = G / 8 / KS;             // one instruction covers 8 codebooks (this wave's share of a slice)
+    constexpr int IWORDS = G / 8 / KS;             // 32-bit index words per token and slice (8 nibbles each), this wave's
+    constexpr int IWORDS_ALL = G / 8;
     constexpr int NBLK = SLICE / 1024;             // 1 KB blocks (one copy instruction of a wave) per slice
     constexpr int DMA_PER_WAVE = (NBLK + SP_WAVES - 1) / SP_WAVES;
     static_assert(KSTEPS >= 2, "the operand pipeline below re-arms inside a slice");
@@ -138,8 +145,8 @@ __global__ __launch_bounds__(NW * 64, sp_wgs_per_cu(TM, NW) * NW / 4 /* waves pe
     constexpr uint32_t POS0 = sp_value_table_bytes(WIDE);  // position words
     constexpr uint32_t BUF0 = sp_table_bytes(WIDE);
     constexpr uint32_t IBUF0 = BUF0 + NBUF * SLICE;
-    constexpr uint32_t IBYTES = sp_ix_blocks(TM, NW) * 64 * 4 * IWORDS;   // index bytes of one slice (64-token blocks)
-    constexpr uint32_t IWAVE = 64 * 4 * IWORDS;               // ... of one wave's 64 tokens
+    constexpr uint32_t IBYTES = sp_ix_blocks(TM, NWT) * 64 * 4 * IWORDS_ALL;   // index bytes of one slice (64-token blocks)
+    constexpr uint32_t IWAVE = 64 * 4 * IWORDS_ALL;           // ... of one 64-token block
     // index words: one operation copies one word of 64 tokens (64 lanes x 4 B) or, where a slice has a multiple of
     // four words, four of them (64 lanes x 16 B: consecutive words of a 64-token block are consecutive 256-byte
     // pieces in the tiled index buffer and in LDS alike); fewer instructions, the same time (measured)
@@ -154,6 +161,8 @@ __global__ __launch_bounds__(NW * 64, sp_wgs_per_cu(TM, NW) * NW / 4 /* waves pe
 
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t tw = KS == 1 ? wave : wave % NWT;  // which tokens of the item
+    const uint32_t kh = KS == 1 ? 0u : wave / NWT;    // which part of a slice's codebooks
     const uint32_t j = lane & 15;  // token within a group (sparse operand) / column within a group (dense operand, result)
     const uint32_t g = lane >> 4;
     if (blockIdx.x >= n_items) return;  // whole workgroup
@@ -192,11 +201,11 @@ __global__ __launch_bounds__(NW * 64, sp_wgs_per_cu(TM, NW) * NW / 4 /* waves pe
     auto locate_lut = [&]() { dma_base = lut + (size_t)col_of(lut_item) * CB_pad * (WN * 16); };
     const uint32_t last_block = (N - 1) / 64;
     auto locate_ix = [&]() {
-        uint32_t blk = (tok_tile_of(ix_item) * TOK_ITEM + wave * (TM * 16)) / 64;
+        uint32_t blk = (tok_tile_of(ix_item) * TOK_ITEM + tw * (TM * 16)) / 64;
         if (blk > last_block) blk = last_block;  // clamp: results of such tokens are never stored
         const uint32_t op = ep.op_col_tiles ? col_of(ix_item) / ep.op_col_tiles : 0u;
         ix_base = idx + (size_t)op * ep.op_idx_stride + (size_t)blk * idx_row_bytes * 64;
-        ix_lane_off = lane * (IX_WIDE ? 16 : 4);
+        ix_lane_off = lane * (IX_WIDE ? 16 : 4) + kh * (IWORDS * 256);  // this wave's words of the block
     };
     // A wave copies DMA_PER_WAVE consecutive 1 KB blocks of a slice.  All of a slice's operations share one
     // global address (the wave's part of the slice, per lane) and one LDS address; the block is chosen by the
@@ -241,7 +250,7 @@ __global__ __launch_bounds__(NW * 64, sp_wgs_per_cu(TM, NW) * NW / 4 /* waves pe
     auto ix_begin = [&](uint32_t ibuf_off, bool fetch) {
         const uint8_t* base = uniform_ptr(fetch ? ix_base : idx);  // idx itself: any 64 tokens' words, never read
         ix_src = base + ix_lane_off;
-        ix_dst = IBUF0 + ibuf_off + (wave * (TM * 16) / 64) * IWAVE;
+        ix_dst = IBUF0 + ibuf_off + (tw * (TM * 16) / 64) * IWAVE + kh * (IWORDS * 256);
     };
     auto ix_op = [&](auto ic) {
         constexpr int i = decltype(ic)::value;
@@ -253,7 +262,7 @@ __global__ __launch_bounds__(NW * 64, sp_wgs_per_cu(TM, NW) * NW / 4 /* waves pe
                                              (__attribute__((address_space(3))) void*)(smem + ix_dst), 4, 256 * i, 0);
     };
     auto ix_advance = [&]() {
-        ix_base += IWORDS * 256;
+        ix_base += IWORDS_ALL * 256;
         if (++ix_s == nslices) {
             ix_s = 0;
             ix_item += gridDim.x;
@@ -268,7 +277,7 @@ __global__ __launch_bounds__(NW * 64, sp_wgs_per_cu(TM, NW) * NW / 4 /* waves pe
     // Index word k of a token holds the nibbles of codebooks 8k .. 8k+7 of the slice; this lane's two are byte g,
     // which it reads on its own (the four lane groups read the four bytes of the same word: one bank, broadcast).
     // Kept as the two table offsets, nibble * 16.
-    const uint32_t ix_lane = IBUF0 + (wave * (TM * 16) / 64) * IWAVE + (((wave * (TM * 16)) & 63) + j) * 4 + g;
+    const uint32_t ix_lane = IBUF0 + (tw * (TM * 16) / 64) * IWAVE + kh * (IWORDS * 256) + (((tw * (TM * 16)) & 63) + j) * 4 + g;
     auto read_ix = [&](uint32_t (&raw)[TM][IWORDS], uint32_t ibuf_off) {
         const uint32_t addr = ix_lane + ibuf_off;
         static_for<0, TM * IWORDS>([&](auto ec) {
@@ -305,7 +314,7 @@ __global__ __launch_bounds__(NW * 64, sp_wgs_per_cu(TM, NW) * NW / 4 /* waves pe
         Epilogue epl = ep;
         if (ep.op_col_tiles) epl.scale = scalar_load1(ep.op_scales + colblk / ep.op_col_tiles);
         const uint32_t tile_tok0 = tok_tile_of(item) * TOK_ITEM;
-        const uint32_t tok0 = tile_tok0 + wave * (TM * 16) + 4 * ge;
+        const uint32_t tok0 = tile_tok0 + tw * (TM * 16) + 4 * ge;
         const bool vec_ok = (M % 4 == 0);
         const bool full = vec_ok && !acc_out && tile_tok0 + TOK_ITEM <= N && (colblk + 1) * WN <= M;
         auto piece = [&](auto c0c, auto wc) __attribute__((always_inline)) {
@@ -383,7 +392,8 @@ __global__ __launch_bounds__(NW * 64, sp_wgs_per_cu(TM, NW) * NW / 4 /* waves pe
     wait_ix(iw_raw);
 
     uint32_t item0 = blockIdx.x;
-    const uint32_t b_lane = BUF0 + (g * WN + j) * 16;  // this lane's 16 bytes of codebook g, column position j
+    // this lane's 16 bytes of codebook g (of this wave's share of the slice), column position j
+    const uint32_t b_lane = BUF0 + (g * WN + j) * 16 + kh * (KSTEPS * 8 * WN * 16);
     // byte offsets of the buffers in their rings: the slice being read and the one its copies go into (the
     // slice before), the index words read next and the ones copied into
     uint32_t cur_off = 0, copy_off = (NBUF - 1) * SLICE, ixn_off = IBYTES, ixc_off = 0;
@@ -498,18 +508,43 @@ __global__ __launch_bounds__(NW * 64, sp_wgs_per_cu(TM, NW) * NW / 4 /* waves pe
         ixc_off = ixn_off;
         ixn_off = ixn_off + IBYTES == NIBUF * IBYTES ? 0 : ixn_off + IBYTES;
     }
-    stores_behind = epilogue(item0);
+    if constexpr (KS == 2) {
+        // the two halves of every sum meet in the slice buffer read last (nothing is copied into it before the next
+        // slice's barrier): waves 4..7 put their accumulators there, waves 0..3 add them to their own
+        static_assert(NWT * 64 * TM * TN * 16 <= SLICE, "the accumulators of half the waves fit a slice buffer");
+        v4i* cbuf = reinterpret_cast<v4i*>(smem + BUF0 + copy_off) + tw * (TM * TN * 64) + lane;
+        __syncthreads();  // every wave is done reading that buffer
+        if (kh == 1) {
+#pragma unroll
+            for (int t = 0; t < TM; ++t)
+#pragma unroll
+                for (int c = 0; c < TN; ++c) {
+                    cbuf[(t * TN + c) * 64] = acc[t][c];
+                    acc[t][c] = (v4i){0, 0, 0, 0};
+                }
+        }
+        __syncthreads();
+        if (kh == 0) {
+#pragma unroll
+            for (int t = 0; t < TM; ++t)
+#pragma unroll
+                for (int c = 0; c < TN; ++c) acc[t][c] += cbuf[(t * TN + c) * 64];
+            stores_behind = epilogue(item0);
+        }
+    } else {
+        stores_behind = epilogue(item0);
+    }
     }
 }
 
-template <int TN, int TM, int GS, int NW = 4, bool WIDE = false>
+template <int TN, int TM, int GS, int NW = 4, bool WIDE = false, int KS = 1>
 int launch_sparse_tm(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out, int32_t* d_acc, uint32_t n,
                      const Epilogue& ep)
 {
-    constexpr int LDS = sp_lds_bytes_tm(TN, TM, GS, NW, WIDE);
+    constexpr int LDS = sp_lds_bytes_tm(TN, TM, GS, NW, WIDE, KS);
     static_assert(sp_wgs_per_cu(TM, NW) * LDS <= 160 * 1024, "the CU's LDS holds the workgroups that its registers hold");
-    constexpr int TOK_ITEM = sp_tok_item(TM, NW);
-    auto kern = gather_sparse_kernel<TN, TM, GS, NW, WIDE>;
+    constexpr int TOK_ITEM = sp_tok_item(TM, NW / KS);
+    auto kern = gather_sparse_kernel<TN, TM, GS, NW, WIDE, KS>;
     const uint32_t cb16 = sparse_codebooks(a.g);  // codebooks of 16 centroids in the tiled table
     if (int rc = allow_dynamic_lds(ctx, reinterpret_cast<const void*>(kern), LDS, "hipFuncSetAttribute(gather_sparse)")) return rc;
     const uint32_t n_token_tiles = (n + TOK_ITEM - 1) / TOK_ITEM;
@@ -518,7 +553,8 @@ int launch_sparse_tm(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out,
     if (grid > n_items) grid = n_items;
     const XcdMap xmap = choose_xcd_map(a.g.M_pad / (16 * TN), n_token_tiles, grid, (uint64_t)cb16 * 16 * a.g.M_pad,
                                        (uint64_t)n * a.g.idx_row_bytes, a.g.tune_xcd_col_split);
-    snprintf(a.last_gather, sizeof(a.last_gather), "gather_sparse_kernel<%d, %d, %d, %d, %s>", TN, TM, GS, NW, WIDE ? "true" : "false");
+    if (KS == 1) snprintf(a.last_gather, sizeof(a.last_gather), "gather_sparse_kernel<%d, %d, %d, %d, %s>", TN, TM, GS, NW, WIDE ? "true" : "false");
+    else snprintf(a.last_gather, sizeof(a.last_gather), "gather_sparse_kernel<%d, %d, %d, %d, %s, %d>", TN, TM, GS, NW, WIDE ? "true" : "false", KS);
     a.note_launch(GS, LDS, TOK_ITEM, NW * 64);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), LDS, ctx->stream, d_idx, reinterpret_cast<const int8_t*>(a.d_lut),
                        d_out, d_acc, n, a.g.M, cb16, a.g.idx_row_bytes, n_token_tiles, n_items, ep, xmap);
@@ -550,6 +586,15 @@ int launch_sparse_tn(Ctx* ctx, const Amm& a, const uint8_t* d_idx, float* d_out,
         if (!a.g.tune_token_item && !a.g.tune_cb_per_slice && cb16 % 64 == 0 && !small_items && items8 >= cus &&
             0.96 * (double)((items8 + cus - 1) / cus) < grid_rounds(items4, slots))
             return launch_sparse_tm<TN, 4, 64, 8>(ctx, a, d_idx, d_out, d_acc, n, ep);
+        // A launch of long sums that offers about one 256-token item per CU: 128-token items would fill the chip's
+        // workgroup slots but copy every slice twice as often and re-read every table entry for two token groups
+        // instead of four; with the codebooks of a slice split between the two waves of a SIMD the 256-token item
+        // keeps both (3072 -> 768: N = 4096 26.3 -> 23.1 us, N = 3072 24.6 -> 22.6; half a round of such items
+        // (N = 2048) or more than one (N = 6144), and sums of 192 codebooks, are not faster that way).
+        if ((a.g.tune_token_item == 256 && a.g.tune_cb_per_slice == 64 && cb16 % 64 == 0) ||
+            (!a.g.tune_token_item && !a.g.tune_cb_per_slice && cb16 % 64 == 0 && cb16 >= 384 && items4 <= cus &&
+             10 * items4 >= 7 * cus))
+            return launch_sparse_tm<TN, 4, 64, 8, false, 2>(ctx, a, d_idx, d_out, d_acc, n, ep);
     }
     if constexpr (!WIDE) if (a.g.tune_token_item == 512) {  // one workgroup of eight waves per CU
         if constexpr (TN == 3) {

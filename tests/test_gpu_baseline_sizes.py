@@ -117,6 +117,37 @@ def test_byte_adder_with_four_token_groups_on_a_ragged_batch(env, C):
     amm.close()
 
 
+@pytest.mark.parametrize("N", [4096, 3800])
+def test_codebook_split_between_the_waves_of_a_simd(env, N):
+    """3072 -> 768 at the 12-layer forward's batch (32 x 128 tokens) and a ragged one: about one 256-token item per
+    CU, which the sparse gather runs with the codebooks of every slice split between the two waves of a SIMD and the
+    halves of each sum added through LDS.  Rows of every token tile's edges and a sample, against the oracle."""
+    pimdl, ctx = env
+    K, v, C, M = 3072, 4, 16, 768
+    rng = np.random.default_rng(1700 + N)
+    CB = K // v
+    x = rng.standard_normal((N, K)).astype(np.float32)
+    cent = rng.standard_normal((CB, C, v)).astype(np.float32)
+    lut = rng.integers(-128, 128, (CB, C, M)).astype(np.int8)
+    bias = rng.standard_normal(M).astype(np.float32)
+    amm = ctx.amm(cent, lut, np.float32(0.0123), bias, max_n=N)
+    out, idx, acc = amm.run_debug(x)
+    if not kernel_switches() and ctx.device_info()["compute_units"] == 256:
+        assert amm.last_gather_kernel().endswith(", 8, false, 2>"), amm.last_gather_kernel()
+    rows = np.unique(np.concatenate([np.arange(0, 70), np.arange(250, 262), np.arange(N - 300, N),
+                                     rng.choice(N, size=64, replace=False)]))
+    w_out, w_idx, w_acc = oracle.amm_cpu(x[rows], cent, lut, bias, v, 0.0123, 0.0, threads=THREADS)
+    assert np.array_equal(idx[rows], w_idx)
+    assert np.array_equal(acc[rows], w_acc)
+    assert np.array_equal(out[rows].view(np.uint32), w_out.view(np.uint32))
+    assert np.array_equal(amm.run(x).view(np.uint32), out.view(np.uint32))  # the launch without the accumulator copy
+    # the same operator told to take 128-token items gives the same bits
+    other = ctx.amm(cent, lut, np.float32(0.0123), bias, max_n=N, tuning={"token_item": 128})
+    assert np.array_equal(other.run(x).view(np.uint32), out.view(np.uint32))
+    other.close()
+    amm.close()
+
+
 @pytest.mark.parametrize("K,M", [(1024, 3072), (1024, 1024), (1024, 4096), (4096, 1024)])
 def test_bert_large_linears_full_batch(env, K, M):
     """BERT-large: hidden 1024, FFN 4096, N = 8192 (fused QKV, O, FFN1, FFN2), v = 4, C = 16."""
